@@ -1,0 +1,80 @@
+// The device layer the engine is written against, bound to the HIP runtime.
+//
+// The engine, the pool and the loopback transport are templates over a
+// "backend" that supplies streams, events, device memory, an asynchronous copy
+// and the segment kernel.  The shipped library instantiates them with
+// HipBackend only; there is no host execution path in it.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "reduce_kernels.hpp"
+#include "status.hpp"
+
+namespace ibcomm_hip {
+
+#define IBCOMM_HIP_CHECK(cmd)                                                                  \
+  do {                                                                                         \
+    hipError_t _e = (cmd);                                                                     \
+    if (_e != hipSuccess)                                                                      \
+      return ::ibcomm_hip::Fail(::ibcomm_hip::kDeviceError, "%s failed at %s:%d: %s", #cmd, __FILE__, __LINE__, \
+                                hipGetErrorString(_e));                                        \
+  } while (0)
+
+struct HipBackend {
+  using Stream = hipStream_t;
+  using Event = hipEvent_t;
+
+  static int Malloc(void** p, size_t bytes) {
+    IBCOMM_HIP_CHECK(hipMalloc(p, bytes));
+    return kOk;
+  }
+  static int Free(void* p) {
+    IBCOMM_HIP_CHECK(hipFree(p));
+    return kOk;
+  }
+  // Pool streams do not synchronise with the legacy default stream
+  // (the reference creates them with cudaStreamNonBlocking, memory_pool.h:96).
+  static int StreamCreate(Stream* s) {
+    IBCOMM_HIP_CHECK(hipStreamCreateWithFlags(s, hipStreamNonBlocking));
+    return kOk;
+  }
+  static int StreamDestroy(Stream s) {
+    IBCOMM_HIP_CHECK(hipStreamDestroy(s));
+    return kOk;
+  }
+  static int StreamSynchronize(Stream s) {
+    IBCOMM_HIP_CHECK(hipStreamSynchronize(s));
+    return kOk;
+  }
+  static int EventCreate(Event* e) {
+    IBCOMM_HIP_CHECK(hipEventCreateWithFlags(e, hipEventDisableTiming));
+    return kOk;
+  }
+  static int EventDestroy(Event e) {
+    IBCOMM_HIP_CHECK(hipEventDestroy(e));
+    return kOk;
+  }
+  static int EventRecord(Event e, Stream s) {
+    IBCOMM_HIP_CHECK(hipEventRecord(e, s));
+    return kOk;
+  }
+  static int StreamWaitEvent(Stream s, Event e) {
+    IBCOMM_HIP_CHECK(hipStreamWaitEvent(s, e, 0));
+    return kOk;
+  }
+  static int EventSynchronize(Event e) {
+    IBCOMM_HIP_CHECK(hipEventSynchronize(e));
+    return kOk;
+  }
+  static int CopyAsync(void* dst, const void* src, size_t bytes, Stream s) {
+    IBCOMM_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
+    return kOk;
+  }
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s) {
+    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, DefaultTuning(), s));
+    return kOk;
+  }
+};
+
+}  // namespace ibcomm_hip

@@ -1,0 +1,591 @@
+// The chunk-pipelined allreduce engine of one emulated rank.
+//
+// Counterpart of IBVerbsCommunicator::AllreduceRingCuda<T> and
+// AllreduceRabenseifnerCuda<T> (ibcomm/allreduce_cuda_impl.h:35-301, 326-717).
+// The reference runs each as a host state machine that polls the network and
+// cudaStreamQuery, and moves every chunk host<->device twice.  Here the whole
+// collective is issued as stream-ordered device work:
+//
+//   * a Plan (plan.hpp) lists, in the reference's wire order, the messages
+//     this rank consumes and emits;
+//   * Progress() walks the plan without ever waiting for the device: it posts
+//     every send whose data has been *enqueued*, takes every message a peer
+//     has posted, lands it in a pool slot (hipMemcpyAsync by default), and
+//     launches one segment kernel over all chunks that landed in this pass:
+//         recvbuf[c] = incoming + sendbuf[c]     ring steps, first halving step
+//         recvbuf[c] = incoming + recvbuf[c]     later halving steps
+//     Finished chunks of the gather phase land straight in recvbuf and are
+//     forwarded from there, so they cost one copy instead of the reference's
+//     three (:129-135, :528-529);
+//   * ordering between ranks, streams and slot reuse is carried by events, so
+//     the same sequence of calls can be recorded into a graph.
+//
+// Summation order is untouched: each element still sees exactly the adds the
+// reference performs, one IEEE add per hop, in the reference's association.
+//
+// A Communicator is driven either by its own thread calling
+// AllreduceBlocking() (one thread per emulated rank, like one process per rank
+// in the reference), or cooperatively by RunWorld() (world.hpp), which steps
+// all ranks from one thread.
+#pragma once
+
+#include <stdint.h>
+#include <string.h>
+
+#include <algorithm>
+#include <chrono>
+#include <deque>
+#include <thread>
+#include <vector>
+
+#include "loopback.hpp"
+#include "memory_pool.hpp"
+#include "plan.hpp"
+#include "segments.hpp"
+#include "status.hpp"
+
+namespace ibcomm_hip {
+
+enum LandingMode : int {
+  kLandMemcpy = 0,  // one asynchronous device copy per message into a pool slot
+  kLandKernel = 1,  // all messages of a pass land through one copy-kernel launch
+  kLandDirect = 2,  // no landing: the reduction reads the sender's buffer in place
+};
+
+struct EngineStats {
+  uint64_t calls = 0;
+  uint64_t reduce_launches = 0;
+  uint64_t reduce_segments = 0;
+  uint64_t reduce_elements = 0;
+  uint64_t landing_copies = 0;  // device copies or copy-kernel launches into pool slots
+  uint64_t landing_bytes = 0;
+  uint64_t gather_copies = 0;   // copies (or copy-kernel launches) of finished chunks into recvbuf
+  uint64_t gather_bytes = 0;
+  uint64_t messages_sent = 0;
+  uint64_t messages_received = 0;
+  uint64_t events_recorded = 0;
+  uint64_t stream_waits = 0;
+  uint64_t streams_created = 0;
+  uint64_t slots_high_water = 0;
+  uint64_t slot_count = 0;
+  uint64_t pool_blocks = 0;
+  uint64_t pool_bytes = 0;
+  uint64_t progress_passes = 0;
+};
+
+template <class B>
+class Communicator {
+ public:
+  using Stream = typename B::Stream;
+  using Event = typename B::Event;
+  using Message = typename Fabric<B>::Message;
+
+  Communicator(Fabric<B>* fabric, int world_size) : fabric_(fabric), world_size_(world_size) {}
+  Communicator(const Communicator&) = delete;
+  Communicator& operator=(const Communicator&) = delete;
+  ~Communicator() {
+    controller_.Release();
+    for (auto& arena : events_)
+      for (auto e : arena) B::EventDestroy(e);
+  }
+
+  // PrepareMemoryPool (ibcomm/ibverbs_communicator_cuda.cpp:26-37) plus this build's knobs.
+  int Init() {
+    if (world_size_ < 1 || world_size_ != fabric_->world_size())
+      return Fail(kInvalidArgument, "world size %d does not match the fabric's %d", world_size_, fabric_->world_size());
+    IBCOMM_RETURN_IF_ERROR(pool_.Init());
+    const char* v = getenv("IBCOMM_HIP_MAX_FUSE");
+    max_fuse_ = v ? atoi(v) : kMaxSegments;
+    if (max_fuse_ < 1 || max_fuse_ > kMaxSegments)
+      return Fail(kInvalidArgument, "IBCOMM_HIP_MAX_FUSE must be in [1, %d]", kMaxSegments);
+    v = getenv("IBCOMM_HIP_LANDING");
+    if (!v || !strcmp(v, "memcpy")) landing_ = kLandMemcpy;
+    else if (!strcmp(v, "kernel")) landing_ = kLandKernel;
+    else if (!strcmp(v, "direct")) landing_ = kLandDirect;
+    else return Fail(kInvalidArgument, "IBCOMM_HIP_LANDING must be memcpy, kernel or direct, not '%s'", v);
+    // The working GPU buffer (IBCOMM_WORK_GPU_MEMORY_SIZE, ibverbs_communicator_cuda.cpp:12-33) held
+    // the second operand of the Rabenseifner kernel.  Here that kernel reads the pool slot itself,
+    // so no such buffer is allocated; the variable is still accepted so job scripts keep working.
+    v = getenv("IBCOMM_WORK_GPU_MEMORY_SIZE");
+    work_gpu_memory_size_ = v ? atoll(v) : (32ll << 20);
+    return kOk;
+  }
+
+  void RegisterMyself(int rank) { rank_ = rank; }  // ibverbs_communicator.cpp:355-357
+  int rank() const { return rank_; }
+  int world_size() const { return world_size_; }
+  MemoryPool<B>& pool() { return pool_; }
+  Fabric<B>* fabric() { return fabric_; }
+  void set_max_fuse(int f) { max_fuse_ = f < 1 ? 1 : (f > kMaxSegments ? kMaxSegments : f); }
+  void set_landing(int mode) { landing_ = mode; }
+  int landing() const { return landing_; }
+  int max_fuse() const { return max_fuse_; }
+  long long work_gpu_memory_size() const { return work_gpu_memory_size_; }
+
+  EngineStats stats() {
+    EngineStats s = stats_;
+    s.streams_created = pool_.streams_created();
+    s.pool_blocks = pool_.blocks();
+    s.pool_bytes = pool_.bytes_allocated();
+    return s;
+  }
+  void reset_stats() { stats_ = EngineStats(); }
+
+  // ---- one collective: Begin, Progress until finished, Finish ------------------------------------
+
+  int Begin(int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len_elements) {
+    if (active_) return Fail(kNotSupported, "an allreduce is already in progress on this communicator");
+    if (rank_ < 0 || rank_ >= world_size_) return Fail(kInvalidArgument, "RegisterMyself has not been called");
+    es_ = DTypeSize(dtype);
+    if (es_ == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+    if (!sendbuf || !recvbuf) return Fail(kInvalidArgument, "sendbuf and recvbuf must not be null");
+    dtype_ = dtype;
+    sendbuf_ = static_cast<const char*>(sendbuf);
+    recvbuf_ = static_cast<char*>(recvbuf);
+    const size_t bytes = len_elements * es_;
+    // The reference's ring cannot run in place (its landing copy overwrites the operand it still
+    // has to add, allreduce_cuda_impl.h:129-133).  This engine can, as long as the two buffers
+    // are the very same range; anything in between is refused.
+    in_place_ = (sendbuf_ == recvbuf_);
+    if (!in_place_ && sendbuf_ < recvbuf_ + bytes && recvbuf_ < sendbuf_ + bytes)
+      return Fail(kInvalidArgument, "sendbuf and recvbuf overlap partially");
+
+    // IBCOMM_CHUNKSIZE is read on every call (ibverbs_communicator.cpp:619-634).
+    IBCOMM_RETURN_IF_ERROR(BuildPlan(algo, world_size_, rank_, len_elements, es_, getenv("IBCOMM_CHUNKSIZE"), &plan_));
+    stats_.calls++;
+    // Events of the call before last are free again: a peer trails this rank by at most one
+    // collective, because finishing a collective needs every peer to have taken part in it.
+    arena_ ^= 1;
+    event_cursor_ = 0;
+    pool_.RewindStreams();
+    next_send_ = next_recv_ = 0;
+    outstanding_sends_ = 0;
+    finished_ = false;
+    pull_events_.clear();
+
+    if (world_size_ == 1) {  // allreduce_cuda_impl.h:40-46
+      if (!in_place_ && bytes) {
+        Stream s;
+        IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(recvbuf_, sendbuf_, bytes, s));
+        stats_.gather_copies++;
+        stats_.gather_bytes += bytes;
+      }
+      finished_ = true;
+      active_ = true;
+      return kOk;
+    }
+
+    const size_t chunks = plan_.part.ranges.size();
+    recv_done_.assign(plan_.recvs.size(), OpState());
+    chunk_last_.assign(chunks, OpState());
+    chunk_unconsumed_.assign(chunks, 0);
+    chunk_pulled_.assign(chunks, OpState());
+    chunk_in_batch_.assign(chunks, 0);
+    posted_.assign(world_size_, std::deque<PostedSend>());
+    pending_reduce_.clear();
+    pending_gather_.clear();
+    IBCOMM_RETURN_IF_ERROR(pool_.GetController(plan_.part.ranges[0].size() * es_, &controller_));
+    active_ = true;
+    return kOk;
+  }
+
+  // Issues everything that can be issued now.  Never waits for the device or for a peer.
+  int Progress(bool* progressed, bool* finished) {
+    *progressed = false;
+    *finished = finished_;
+    if (!active_) return Fail(kInvalidArgument, "Progress without Begin");
+    if (finished_) return kOk;
+    stats_.progress_passes++;
+    for (;;) {
+      bool moved = false;
+      IBCOMM_RETURN_IF_ERROR(DrainSendCompletions(&moved));
+      IBCOMM_RETURN_IF_ERROR(PostSends(&moved));
+      IBCOMM_RETURN_IF_ERROR(TakeMessages(&moved));
+      IBCOMM_RETURN_IF_ERROR(FlushGathers());
+      IBCOMM_RETURN_IF_ERROR(FlushReduces());
+      if (!moved) break;
+      *progressed = true;
+    }
+    finished_ = next_send_ == plan_.sends.size() && next_recv_ == plan_.recvs.size() && outstanding_sends_ == 0;
+    *finished = finished_;
+    return kOk;
+  }
+
+  // Waits for this rank's device work (and, with wait_pulls, for the peers' reads of this rank's
+  // buffers) and releases the pool controller.  The collective is complete for the caller when
+  // this returns, as in the reference (allreduce_cuda_impl.h:280-299, :709-715).
+  int Finish(bool wait_pulls) {
+    if (!active_) return kOk;
+    int rc = pool_.SynchronizeStreams();
+    if (rc == kOk && wait_pulls) {
+      for (Event e : pull_events_) {
+        rc = B::EventSynchronize(e);
+        if (rc != kOk) break;
+      }
+    }
+    ReleaseCall();
+    return rc;
+  }
+
+  // Same as Finish but without touching the device: for a caller that has synchronised already
+  // (or is recording a graph and will synchronise the replay).
+  void FinishNoSync() {
+    if (active_) ReleaseCall();
+  }
+
+  void Abort() {
+    if (!active_) return;
+    pool_.SynchronizeStreams();
+    ReleaseCall();
+  }
+
+  // Per-rank blocking call: the shape of AllreduceRingCuda / AllreduceRabenseifnerCuda.  Every
+  // emulated rank must be inside the same collective on a thread of its own.
+  int AllreduceBlocking(int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len_elements) {
+    IBCOMM_RETURN_IF_ERROR(Begin(algo, dtype, sendbuf, recvbuf, len_elements));
+    const char* t = getenv("IBCOMM_HIP_TIMEOUT_S");
+    const double limit = t ? atof(t) : 120.0;
+    const auto t0 = std::chrono::steady_clock::now();
+    bool progressed = false, finished = false;
+    for (;;) {
+      const int rc = Progress(&progressed, &finished);
+      if (rc != kOk) {
+        Abort();
+        return rc;
+      }
+      if (finished) break;
+      if (!progressed) {
+        std::this_thread::yield();
+        const double waited = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (waited > limit) {
+          Abort();
+          return Fail(kTransportError, "rank %d: no peer progress for %.0f s (recv %zu/%zu, send %zu/%zu)", rank_, limit,
+                      next_recv_, plan_.recvs.size(), next_send_, plan_.sends.size());
+        }
+      }
+    }
+    return Finish(true);
+  }
+
+  const Plan& plan() const { return plan_; }
+  bool active() const { return active_; }
+  size_t recv_cursor() const { return next_recv_; }
+  size_t send_cursor() const { return next_send_; }
+  size_t recv_total() const { return plan_.recvs.size(); }
+  size_t send_total() const { return plan_.sends.size(); }
+
+ private:
+  struct OpState {
+    bool issued = false;     // the device work has been enqueued
+    bool has_event = false;  // ... and `event` completes with it
+    Event event{};
+    Stream stream{};         // stream the event was recorded on (ours), or Stream{} for a peer's
+  };
+  struct PendingRecv {
+    int op = 0;              // index into plan_.recvs
+    Message msg;
+    Memory<B>* slot = nullptr;  // landing slot; null for gathers and in direct mode
+  };
+  struct PostedSend {
+    uint64_t ticket;
+    int send_index;
+  };
+
+  char* RecvPtr(int chunk) const { return recvbuf_ + plan_.part.ranges[chunk].begin * es_; }
+  const char* SendPtr(int chunk) const { return sendbuf_ + plan_.part.ranges[chunk].begin * es_; }
+  size_t ChunkElems(int chunk) const { return plan_.part.ranges[chunk].size(); }
+  size_t ChunkBytes(int chunk) const { return plan_.part.ranges[chunk].size() * es_; }
+
+  void ReleaseCall() {
+    stats_.slots_high_water = std::max<uint64_t>(stats_.slots_high_water, controller_.high_water());
+    if (controller_.active()) stats_.slot_count = controller_.slot_count();
+    controller_.Release();
+    pull_events_.clear();
+    active_ = false;
+  }
+
+  int RecordEvent(Stream s, OpState* st) {
+    std::vector<Event>& arena = events_[arena_];
+    if (event_cursor_ == arena.size()) {
+      Event e;
+      IBCOMM_RETURN_IF_ERROR(B::EventCreate(&e));
+      arena.push_back(e);
+    }
+    st->event = arena[event_cursor_++];
+    st->stream = s;
+    st->has_event = true;
+    st->issued = true;
+    stats_.events_recorded++;
+    return B::EventRecord(st->event, s);
+  }
+
+  // Orders stream s after `st` unless it already is (same stream) or there is nothing to wait for.
+  int WaitOn(Stream s, const OpState& st) {
+    if (!st.has_event || st.stream == s) return kOk;
+    stats_.stream_waits++;
+    return B::StreamWaitEvent(s, st.event);
+  }
+  int WaitOnMessage(Stream s, const Message& m) {
+    if (!m.has_ready) return kOk;
+    stats_.stream_waits++;
+    return B::StreamWaitEvent(s, m.ready);
+  }
+
+  int DrainSendCompletions(bool* moved) {
+    for (int peer = 0; peer < world_size_; peer++) {
+      typename Fabric<B>::Completion c;
+      while (!posted_[peer].empty() && fabric_->PollSendCompletion(rank_, peer, &c)) {
+        const PostedSend ps = posted_[peer].front();
+        posted_[peer].pop_front();
+        if (ps.ticket != c.ticket)
+          return Fail(kTransportError, "rank %d: completion for ticket %llu from rank %d while %llu is the oldest send", rank_,
+                      (unsigned long long)c.ticket, peer, (unsigned long long)ps.ticket);
+        const SendOp& s = plan_.sends[ps.send_index];
+        outstanding_sends_--;
+        if (c.has_done) pull_events_.push_back(c.done);
+        if (s.dep >= 0 || in_place_) {
+          chunk_unconsumed_[s.chunk]--;
+          OpState& p = chunk_pulled_[s.chunk];
+          p.issued = true;
+          p.has_event = c.has_done;
+          p.event = c.done;
+          p.stream = Stream{};
+        }
+        *moved = true;
+      }
+    }
+    return kOk;
+  }
+
+  int PostSends(bool* moved) {
+    while (next_send_ < plan_.sends.size()) {
+      const SendOp& s = plan_.sends[next_send_];
+      const void* src;
+      Event ready{};
+      bool has_ready = false;
+      if (s.dep < 0) {
+        src = SendPtr(s.chunk);
+      } else {
+        const OpState& d = recv_done_[s.dep];
+        if (!d.issued) break;  // the data has not been enqueued yet
+        src = RecvPtr(s.chunk);
+        ready = d.event;
+        has_ready = d.has_event;
+      }
+      const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready);
+      posted_[s.peer].push_back(PostedSend{ticket, static_cast<int>(next_send_)});
+      if (s.dep >= 0 || in_place_) chunk_unconsumed_[s.chunk]++;
+      outstanding_sends_++;
+      stats_.messages_sent++;
+      next_send_++;
+      *moved = true;
+    }
+    return kOk;
+  }
+
+  int TakeMessages(bool* moved) {
+    while (next_recv_ < plan_.recvs.size()) {
+      const RecvOp& r = plan_.recvs[next_recv_];
+      // A gather overwrites recvbuf[chunk]; a send of ours out of that range must have been read first.
+      if (r.kind == kGather && chunk_unconsumed_[r.chunk] > 0) break;
+      PendingRecv p;
+      if (!fabric_->Take(rank_, r.peer, &p.msg)) break;
+      if (p.msg.bytes != ChunkBytes(r.chunk))
+        return Fail(kTransportError, "rank %d: message of %zu bytes from rank %d where chunk %d has %zu", rank_, p.msg.bytes,
+                    r.peer, r.chunk, ChunkBytes(r.chunk));
+      p.op = static_cast<int>(next_recv_);
+      // Completions of a channel go back in the order taken, so the two pending lists never hold
+      // messages at the same time.
+      if (r.kind == kGather) {
+        IBCOMM_RETURN_IF_ERROR(FlushReduces());
+        pending_gather_.push_back(p);
+        if (static_cast<int>(pending_gather_.size()) >= max_fuse_) IBCOMM_RETURN_IF_ERROR(FlushGathers());
+      } else {
+        IBCOMM_RETURN_IF_ERROR(FlushGathers());
+        // Segments of one launch run concurrently: a chunk whose previous partial sum is still
+        // waiting in this batch must go into the next launch.
+        if (chunk_in_batch_[r.chunk]) IBCOMM_RETURN_IF_ERROR(FlushReduces());
+        if (landing_ != kLandDirect) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+        chunk_in_batch_[r.chunk] = 1;
+        pending_reduce_.push_back(p);
+        if (static_cast<int>(pending_reduce_.size()) >= max_fuse_) IBCOMM_RETURN_IF_ERROR(FlushReduces());
+      }
+      next_recv_++;
+      stats_.messages_received++;
+      *moved = true;
+    }
+    return kOk;
+  }
+
+  // Finished chunks: recvbuf[c] <- message.
+  int FlushGathers() {
+    if (pending_gather_.empty()) return kOk;
+    if (landing_ == kLandKernel) {
+      Stream s;
+      IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+      SegmentBatch batch;
+      batch.count = 0;
+      for (const PendingRecv& p : pending_gather_) {
+        const int c = plan_.recvs[p.op].chunk;
+        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
+        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
+        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
+        batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, p.msg.src, nullptr, ChunkElems(c)};
+        stats_.gather_bytes += ChunkBytes(c);
+      }
+      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s));
+      stats_.gather_copies++;
+      OpState done;
+      IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+      for (const PendingRecv& p : pending_gather_) {
+        const RecvOp& r = plan_.recvs[p.op];
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+        recv_done_[p.op] = done;
+        chunk_last_[r.chunk] = done;
+      }
+    } else {
+      for (const PendingRecv& p : pending_gather_) {
+        const RecvOp& r = plan_.recvs[p.op];
+        const int c = r.chunk;
+        Stream s;
+        IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
+        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
+        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
+        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(RecvPtr(c), p.msg.src, ChunkBytes(c), s));
+        stats_.gather_copies++;
+        stats_.gather_bytes += ChunkBytes(c);
+        OpState done;
+        IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+        recv_done_[p.op] = done;
+        chunk_last_[c] = done;
+      }
+    }
+    pending_gather_.clear();
+    return kOk;
+  }
+
+  // Partial sums: land every pending message, then one launch adds them all.
+  int FlushReduces() {
+    if (pending_reduce_.empty()) return kOk;
+    const size_t n = pending_reduce_.size();
+    Stream s{};
+    std::vector<OpState> landed(n);
+
+    if (landing_ == kLandMemcpy) {
+      for (size_t i = 0; i < n; i++) {
+        PendingRecv& p = pending_reduce_[i];
+        const RecvOp& r = plan_.recvs[p.op];
+        Stream si;
+        IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&si));
+        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(si, p.msg));
+        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(si, p.slot));
+        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(p.slot->LandingFor(RecvPtr(r.chunk)), p.msg.src, ChunkBytes(r.chunk), si));
+        stats_.landing_copies++;
+        stats_.landing_bytes += ChunkBytes(r.chunk);
+        IBCOMM_RETURN_IF_ERROR(RecordEvent(si, &landed[i]));
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, landed[i].event, true);
+      }
+      s = landed[0].stream;
+      for (size_t i = 1; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOn(s, landed[i]));
+    } else {
+      IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+      for (size_t i = 0; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, pending_reduce_[i].msg));
+      if (landing_ == kLandKernel) {
+        SegmentBatch copy;
+        copy.count = 0;
+        for (size_t i = 0; i < n; i++) {
+          PendingRecv& p = pending_reduce_[i];
+          const int c = plan_.recvs[p.op].chunk;
+          IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.slot));
+          copy.seg[copy.count++] = Segment{p.slot->LandingFor(RecvPtr(c)), nullptr, p.msg.src, nullptr, ChunkElems(c)};
+          stats_.landing_bytes += ChunkBytes(c);
+        }
+        IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s));
+        stats_.landing_copies++;
+        OpState done;
+        IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+        for (size_t i = 0; i < n; i++) {
+          const PendingRecv& p = pending_reduce_[i];
+          fabric_->Complete(rank_, plan_.recvs[p.op].peer, p.msg.ticket, done.event, true);
+        }
+      }
+    }
+
+    SegmentBatch batch;
+    batch.count = 0;
+    for (size_t i = 0; i < n; i++) {
+      const PendingRecv& p = pending_reduce_[i];
+      const RecvOp& r = plan_.recvs[p.op];
+      const int c = r.chunk;
+      const void* incoming = (landing_ == kLandDirect) ? p.msg.src : p.slot->LandingFor(RecvPtr(c));
+      const void* own;
+      if (r.kind == kReduceWithSendbuf) {
+        own = SendPtr(c);
+      } else {
+        own = RecvPtr(c);
+        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));  // the previous halving step's sum
+      }
+      batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, incoming, own, ChunkElems(c)};
+      stats_.reduce_elements += ChunkElems(c);
+    }
+    IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s));
+    stats_.reduce_launches++;
+    stats_.reduce_segments += n;
+    OpState done;
+    IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+    for (size_t i = 0; i < n; i++) {
+      const PendingRecv& p = pending_reduce_[i];
+      const RecvOp& r = plan_.recvs[p.op];
+      recv_done_[p.op] = done;
+      chunk_last_[r.chunk] = done;
+      if (p.slot) controller_.returnMemory(p.slot, done.event, s);
+      if (landing_ == kLandDirect) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+      chunk_in_batch_[r.chunk] = 0;
+    }
+    pending_reduce_.clear();
+    return kOk;
+  }
+
+  int WaitOnSlot(Stream s, const Memory<B>* slot) {
+    if (!slot->has_free_event || slot->free_stream == s) return kOk;
+    stats_.stream_waits++;
+    return B::StreamWaitEvent(s, slot->free_event);
+  }
+
+  Fabric<B>* fabric_;
+  int world_size_;
+  int rank_ = -1;
+  MemoryPool<B> pool_;
+  MemoryController<B> controller_;
+  int max_fuse_ = kMaxSegments;
+  int landing_ = kLandMemcpy;
+  long long work_gpu_memory_size_ = 0;
+
+  bool active_ = false;
+  bool finished_ = false;
+  bool in_place_ = false;
+  Plan plan_;
+  int dtype_ = kF32;
+  size_t es_ = 4;
+  const char* sendbuf_ = nullptr;
+  char* recvbuf_ = nullptr;
+  size_t next_send_ = 0, next_recv_ = 0;
+  size_t outstanding_sends_ = 0;
+  std::vector<OpState> recv_done_;        // per receive op: result enqueued (+ completion event)
+  std::vector<OpState> chunk_last_;       // per chunk: our last device op that wrote recvbuf[chunk]
+  std::vector<int> chunk_unconsumed_;     // per chunk: our sends out of recvbuf[chunk] no peer has taken yet
+  std::vector<OpState> chunk_pulled_;     // per chunk: the peer's latest read of recvbuf[chunk]
+  std::vector<char> chunk_in_batch_;      // per chunk: a reduction of it sits in pending_reduce_
+  std::vector<std::deque<PostedSend>> posted_;  // per peer: sends awaiting completion, oldest first
+  std::vector<PendingRecv> pending_reduce_, pending_gather_;
+  std::vector<Event> pull_events_;
+  std::vector<Event> events_[2];
+  int arena_ = 0;
+  size_t event_cursor_ = 0;
+  EngineStats stats_;
+};
+
+}  // namespace ibcomm_hip

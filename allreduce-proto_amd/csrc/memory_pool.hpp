@@ -1,0 +1,251 @@
+// Staging memory and streams for the chunk pipelines, resident in HBM.
+//
+// Role of the reference's MemoryPool / MemoryController / MemoryBlock / Memory
+// (ibcomm/memory_pool.h:28-283, memory_pool.cpp:11-55): pre-allocated blocks
+// carved into chunk-sized slots that incoming messages land in, plus the pool
+// of streams the per-chunk work is issued on, both handed out first-in
+// first-out.  Differences that come from living on one MI355X:
+//
+//   * blocks are device memory (hipMalloc), not pinned host memory registered
+//     with an HCA; nothing crosses PCIe;
+//   * a slot is handed back as soon as the kernel that reads it has been
+//     *enqueued*, together with the event that marks that kernel's completion;
+//     the next user of the slot orders itself after that event on the device.
+//     The host never waits for a slot, so a handful of slots sustain the whole
+//     pipeline and the pool does not grow with the buffer;
+//   * each slot keeps 16 spare bytes so that a message can land at the same
+//     16-byte phase as the recvbuf range it will be added to, which keeps the
+//     kernel's body on dwordx4 accesses for odd chunk offsets;
+//   * carving uses every slot that fits ((i + 1) * stride <= block) where the
+//     reference's strict '<' (memory_pool.h:269) leaves the last one unused,
+//     and a chunk larger than a block makes the pool allocate a block that
+//     fits two chunks instead of handing out memory it does not have
+//     (memory_pool.h:229-233);
+//   * IBCOMM_MEMORY_POOL_PRE_ALLOC is read as a 64-bit value without the
+//     reference's 1 GiB ceiling (memory_pool.h:163), default 256 MiB;
+//     IBCOMM_NUM_CUDA_STREAM keeps its name and its (0, 1024] range
+//     (memory_pool.h:139-154); streams are created on first use and the
+//     default is 8, because a process drives 4 hardware queues on this GPU.
+#pragma once
+
+#include <stdlib.h>
+
+#include <deque>
+#include <memory>
+#include <vector>
+
+#include "status.hpp"
+
+namespace ibcomm_hip {
+
+template <class B>
+struct Memory {
+  char* base = nullptr;            // 256-byte aligned start of the slot
+  size_t capacity = 0;             // usable bytes including the phase margin
+  typename B::Event free_event{};  // valid iff has_free_event: last reader's completion
+  bool has_free_event = false;
+  typename B::Stream free_stream{};  // stream free_event was recorded on
+  // Where a message bound for `target` should land so that both share their 16-byte phase.
+  char* LandingFor(const void* target) const { return base + (reinterpret_cast<uintptr_t>(target) & 15); }
+};
+
+template <class B>
+class MemoryPool;
+
+template <class B>
+class MemoryController {
+ public:
+  MemoryController() = default;
+  MemoryController(const MemoryController&) = delete;
+  MemoryController& operator=(const MemoryController&) = delete;
+  ~MemoryController() { Release(); }
+
+  bool active() const { return pool_ != nullptr; }
+  size_t slot_count() const { return slots_.size(); }
+  int held() const { return held_; }
+  int high_water() const { return high_water_; }
+
+  // FIFO hand-out (memory_pool.h:222-236).  Grows the pool by one block if no slot is vacant.
+  int getMemory(Memory<B>** out);
+  // FIFO return (memory_pool.h:238-242); `after` completes when the slot's contents are dead.
+  void returnMemory(Memory<B>* m, typename B::Event after, typename B::Stream stream) {
+    m->free_event = after;
+    m->free_stream = stream;
+    m->has_free_event = true;
+    vacant_.push_back(m);
+    held_--;
+  }
+  void returnMemory(Memory<B>* m) {
+    vacant_.push_back(m);
+    held_--;
+  }
+  void Release();
+
+ private:
+  friend class MemoryPool<B>;
+  void Carve(char* block, size_t block_bytes);
+
+  MemoryPool<B>* pool_ = nullptr;
+  size_t stride_ = 0;
+  std::vector<std::unique_ptr<Memory<B>>> slots_;
+  std::deque<Memory<B>*> vacant_;
+  int held_ = 0;
+  int high_water_ = 0;
+};
+
+template <class B>
+class MemoryPool {
+ public:
+  static constexpr int kDefaultNumStreams = 8;
+  static constexpr size_t kDefaultPreAlloc = size_t(256) << 20;
+
+  MemoryPool() = default;
+  MemoryPool(const MemoryPool&) = delete;
+  MemoryPool& operator=(const MemoryPool&) = delete;
+  ~MemoryPool() { Destroy(); }
+
+  // Reads the knobs and allocates the first block (memory_pool.h:86-100).
+  int Init() {
+    IBCOMM_RETURN_IF_ERROR(ReadNumStreams(&max_streams_));
+    IBCOMM_RETURN_IF_ERROR(ReadPreAlloc(&block_bytes_));
+    return AllocateBlock(block_bytes_, nullptr);
+  }
+
+  void Destroy() {
+    for (auto s : streams_) B::StreamDestroy(s);
+    streams_.clear();
+    for (auto& b : blocks_) B::Free(b.first);
+    blocks_.clear();
+  }
+
+  // One controller at a time (memory_pool.h:111-121).
+  int GetController(size_t chunk_bytes, MemoryController<B>* c) {
+    if (controller_in_use_) return Fail(kNotSupported, "Currently, MemoryController is in use.");
+    if (chunk_bytes == 0) return Fail(kInvalidArgument, "chunk size must be positive");
+    controller_in_use_ = true;
+    c->pool_ = this;
+    c->stride_ = (chunk_bytes + 16 + 255) & ~size_t(255);
+    c->slots_.clear();
+    c->vacant_.clear();
+    c->held_ = 0;
+    c->high_water_ = 0;
+    for (auto& b : blocks_) c->Carve(b.first, b.second);
+    return kOk;
+  }
+
+  // Round-robin over at most max_streams() streams, created on first use.
+  int NextStream(typename B::Stream* out) {
+    if (static_cast<int>(streams_.size()) < max_streams_ && cursor_ >= streams_.size()) {
+      typename B::Stream s;
+      IBCOMM_RETURN_IF_ERROR(B::StreamCreate(&s));
+      streams_.push_back(s);
+    }
+    if (cursor_ >= streams_.size()) cursor_ = 0;
+    *out = streams_[cursor_++];
+    return kOk;
+  }
+  void RewindStreams() { cursor_ = 0; }
+
+  int SynchronizeStreams() {
+    for (auto s : streams_) IBCOMM_RETURN_IF_ERROR(B::StreamSynchronize(s));
+    return kOk;
+  }
+
+  int max_streams() const { return max_streams_; }
+  size_t streams_created() const { return streams_.size(); }
+  const std::vector<typename B::Stream>& streams() const { return streams_; }
+  size_t block_bytes() const { return block_bytes_; }
+  size_t blocks() const { return blocks_.size(); }
+  size_t bytes_allocated() const {
+    size_t t = 0;
+    for (auto& b : blocks_) t += b.second;
+    return t;
+  }
+
+ private:
+  friend class MemoryController<B>;
+
+  static int ReadNumStreams(int* out) {
+    const char* v = getenv("IBCOMM_NUM_CUDA_STREAM");
+    if (!v) {
+      *out = kDefaultNumStreams;
+      return kOk;
+    }
+    const int n = atoi(v);
+    if (n <= 0 || n > 1024) return Fail(kInvalidArgument, "Invalid value for IBCOMM_NUM_CUDA_STREAM: %s", v);
+    *out = n;
+    return kOk;
+  }
+
+  static int ReadPreAlloc(size_t* out) {
+    const char* v = getenv("IBCOMM_MEMORY_POOL_PRE_ALLOC");
+    if (!v) {
+      *out = kDefaultPreAlloc;
+      return kOk;
+    }
+    const long long n = atoll(v);
+    if (n < 4) return Fail(kInvalidArgument, "Invalid value for IBCOMM_MEMORY_POOL_PRE_ALLOC: %s", v);
+    *out = static_cast<size_t>(n);
+    return kOk;
+  }
+
+  int AllocateBlock(size_t bytes, char** out) {
+    void* p = nullptr;
+    IBCOMM_RETURN_IF_ERROR(B::Malloc(&p, bytes));
+    blocks_.emplace_back(static_cast<char*>(p), bytes);
+    if (out) *out = static_cast<char*>(p);
+    return kOk;
+  }
+
+  void CompleteMemoryController() { controller_in_use_ = false; }
+
+  int max_streams_ = kDefaultNumStreams;
+  size_t block_bytes_ = kDefaultPreAlloc;
+  std::vector<std::pair<char*, size_t>> blocks_;
+  std::vector<typename B::Stream> streams_;
+  size_t cursor_ = 0;
+  bool controller_in_use_ = false;
+};
+
+template <class B>
+void MemoryController<B>::Carve(char* block, size_t block_bytes) {
+  // Slots are reused first-in first-out and a pass holds at most one launch's worth of them, so
+  // beyond a few hundred more slots buy nothing; tiny chunks would otherwise yield millions.
+  constexpr size_t kMaxSlotsPerBlock = 1024;
+  for (size_t i = 0; (i + 1) * stride_ <= block_bytes && i < kMaxSlotsPerBlock; i++) {
+    slots_.emplace_back(new Memory<B>());
+    Memory<B>* m = slots_.back().get();
+    m->base = block + i * stride_;
+    m->capacity = stride_;
+    vacant_.push_back(m);
+  }
+}
+
+template <class B>
+int MemoryController<B>::getMemory(Memory<B>** out) {
+  if (!pool_) return Fail(kInvalidArgument, "MemoryController is not attached to a pool");
+  if (vacant_.empty()) {
+    size_t bytes = pool_->block_bytes();
+    if (bytes < 2 * stride_) bytes = 2 * stride_;
+    char* block = nullptr;
+    IBCOMM_RETURN_IF_ERROR(pool_->AllocateBlock(bytes, &block));
+    Carve(block, bytes);
+  }
+  Memory<B>* m = vacant_.front();
+  vacant_.pop_front();
+  held_++;
+  if (held_ > high_water_) high_water_ = held_;
+  *out = m;
+  return kOk;
+}
+
+template <class B>
+void MemoryController<B>::Release() {
+  if (!pool_) return;
+  slots_.clear();
+  vacant_.clear();
+  pool_->CompleteMemoryController();
+  pool_ = nullptr;
+}
+
+}  // namespace ibcomm_hip

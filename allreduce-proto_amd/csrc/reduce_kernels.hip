@@ -1,0 +1,208 @@
+// gfx950 streaming add / copy kernels.  See reduce_kernels.hpp for the contract.
+#include "reduce_kernels.hpp"
+
+#include <stdlib.h>
+
+namespace ibcomm_hip {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+
+template <bool NT, typename V>
+__device__ __forceinline__ V LoadVec(const V* p) {
+  if (NT) return __builtin_nontemporal_load(p);
+  return *p;
+}
+
+template <bool NT, typename V>
+__device__ __forceinline__ void StoreVec(V* p, V v) {
+  if (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
+// One workgroup column (blockIdx.y) per segment; blockIdx.x strides over tiles
+// of THREADS * UNROLL 16-byte vectors.  T is the element type, V the 16-byte
+// vector of T.  Integer types are instantiated unsigned so that += wraps.
+template <typename T, typename V, int THREADS, int UNROLL, bool NT>
+__global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batch) {
+  const Segment s = batch.seg[blockIdx.y];
+  const uint64_t n = s.n;
+  if (n == 0) return;
+
+  T* dst = static_cast<T*>(s.dst);
+  T* dst2 = static_cast<T*>(s.dst2);
+  const T* a = static_cast<const T*>(s.a);
+  const T* b = static_cast<const T*>(s.b);
+  const bool has_b = (b != nullptr);
+  const bool has_d2 = (dst2 != nullptr);
+
+  constexpr uint64_t kPerVec = 16 / sizeof(T);
+  const uintptr_t pd = reinterpret_cast<uintptr_t>(dst) & 15;
+  const bool same_phase = ((reinterpret_cast<uintptr_t>(a) & 15) == pd) &&
+                          (!has_b || (reinterpret_cast<uintptr_t>(b) & 15) == pd) &&
+                          (!has_d2 || (reinterpret_cast<uintptr_t>(dst2) & 15) == pd) &&
+                          (pd % sizeof(T) == 0);
+
+  // [0, head) scalar, [head, head + nvec * kPerVec) as 16-byte vectors, rest scalar.
+  uint64_t head = n, nvec = 0;
+  if (same_phase) {
+    head = ((16 - pd) & 15) / sizeof(T);
+    if (head > n) head = n;
+    nvec = (n - head) / kPerVec;
+  }
+
+  if (nvec) {
+    const V* av = reinterpret_cast<const V*>(a + head);
+    const V* bv = reinterpret_cast<const V*>(b + head);
+    V* dv = reinterpret_cast<V*>(dst + head);
+    V* d2v = reinterpret_cast<V*>(dst2 + head);
+    constexpr uint64_t kTile = static_cast<uint64_t>(THREADS) * UNROLL;
+    for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kTile; base < nvec;
+         base += static_cast<uint64_t>(gridDim.x) * kTile) {
+      V ra[UNROLL];
+      V rb[UNROLL];
+      if (base + kTile <= nvec) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) ra[u] = LoadVec<NT>(av + base + u * THREADS + threadIdx.x);
+        if (has_b) {
+#pragma unroll
+          for (int u = 0; u < UNROLL; u++) rb[u] = LoadVec<NT>(bv + base + u * THREADS + threadIdx.x);
+#pragma unroll
+          for (int u = 0; u < UNROLL; u++) ra[u] = ra[u] + rb[u];
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) StoreVec<NT>(dv + base + u * THREADS + threadIdx.x, ra[u]);
+        if (has_d2) {
+#pragma unroll
+          for (int u = 0; u < UNROLL; u++) StoreVec<NT>(d2v + base + u * THREADS + threadIdx.x, ra[u]);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+          const uint64_t i = base + u * THREADS + threadIdx.x;
+          if (i < nvec) {
+            V v = LoadVec<NT>(av + i);
+            if (has_b) v = v + LoadVec<NT>(bv + i);
+            StoreVec<NT>(dv + i, v);
+            if (has_d2) StoreVec<NT>(d2v + i, v);
+          }
+        }
+      }
+    }
+  }
+
+  // Scalar remainder: fewer than two vectors' worth when the phases agree,
+  // the whole segment when they do not.
+  const uint64_t tail_begin = head + nvec * kPerVec;
+  const uint64_t scalar_count = head + (n - tail_begin);
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * THREADS;
+  for (uint64_t k = static_cast<uint64_t>(blockIdx.x) * THREADS + threadIdx.x; k < scalar_count; k += stride) {
+    const uint64_t i = (k < head) ? k : tail_begin + (k - head);
+    T v = a[i];
+    if (has_b) v = v + b[i];
+    dst[i] = v;
+    if (has_d2) dst2[i] = v;
+  }
+}
+
+namespace {
+
+template <typename T, typename V, int THREADS, int UNROLL, bool NT>
+hipError_t LaunchOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
+  hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, UNROLL, NT>), grid, dim3(THREADS), 0, stream, batch);
+  return hipGetLastError();
+}
+
+template <typename T, typename V, int THREADS, int UNROLL>
+hipError_t LaunchNT(const SegmentBatch& batch, dim3 grid, bool nt, hipStream_t stream) {
+  return nt ? LaunchOne<T, V, THREADS, UNROLL, true>(batch, grid, stream)
+            : LaunchOne<T, V, THREADS, UNROLL, false>(batch, grid, stream);
+}
+
+template <typename T, typename V, int THREADS>
+hipError_t LaunchUnroll(const SegmentBatch& batch, dim3 grid, int unroll, bool nt, hipStream_t stream) {
+  switch (unroll) {
+    case 1: return LaunchNT<T, V, THREADS, 1>(batch, grid, nt, stream);
+    case 2: return LaunchNT<T, V, THREADS, 2>(batch, grid, nt, stream);
+    case 4: return LaunchNT<T, V, THREADS, 4>(batch, grid, nt, stream);
+    case 8: return LaunchNT<T, V, THREADS, 8>(batch, grid, nt, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <typename T, typename V>
+hipError_t LaunchThreads(const SegmentBatch& batch, dim3 grid, const LaunchTuning& t, hipStream_t stream) {
+  switch (t.threads) {
+    case 256: return LaunchUnroll<T, V, 256>(batch, grid, t.unroll, t.nontemporal, stream);
+    case 512: return LaunchUnroll<T, V, 512>(batch, grid, t.unroll, t.nontemporal, stream);
+    case 1024: return LaunchUnroll<T, V, 1024>(batch, grid, t.unroll, t.nontemporal, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int EnvInt(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
+
+}  // namespace
+
+LaunchTuning DefaultTuning() {
+  // Tunables for experiments; the defaults are what the sweep on MI355X picked.
+  static const LaunchTuning t = {
+      EnvInt("IBCOMM_HIP_THREADS", 256),
+      EnvInt("IBCOMM_HIP_UNROLL", 1),
+      EnvInt("IBCOMM_HIP_MAX_BLOCKS", 0),
+      EnvInt("IBCOMM_HIP_NONTEMPORAL", 1) != 0,
+  };
+  return t;
+}
+
+hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuning& tuning, hipStream_t stream) {
+  if (batch.count <= 0) return hipSuccess;
+  if (batch.count > kMaxSegments) return hipErrorInvalidValue;
+  const size_t es = DTypeSize(dtype);
+  if (es == 0) return hipErrorInvalidValue;
+
+  uint64_t max_n = 0;
+  for (int i = 0; i < batch.count; i++) {
+    const Segment& s = batch.seg[i];
+    if (s.n && (!s.dst || !s.a)) return hipErrorInvalidValue;
+    if (s.n > max_n) max_n = s.n;
+  }
+  if (max_n == 0) return hipSuccess;
+
+  const uint64_t per_vec = 16 / es;
+  const uint64_t tile = static_cast<uint64_t>(tuning.threads) * tuning.unroll;
+  uint64_t blocks = (max_n / per_vec + tile - 1) / tile;
+  if (blocks == 0) blocks = 1;
+  if (tuning.max_blocks_x > 0 && blocks > static_cast<uint64_t>(tuning.max_blocks_x)) blocks = tuning.max_blocks_x;
+  if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
+
+  switch (dtype) {
+    case kF32: return LaunchThreads<float, f32x4>(batch, grid, tuning, stream);
+    case kI32: return LaunchThreads<uint32_t, u32x4>(batch, grid, tuning, stream);
+    case kF64: return LaunchThreads<double, f64x2>(batch, grid, tuning, stream);
+    case kI64: return LaunchThreads<uint64_t, u64x2>(batch, grid, tuning, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t LaunchReduce2(void* dst, const void* a, const void* b, size_t n, int dtype, hipStream_t stream) {
+  SegmentBatch batch;
+  batch.count = 1;
+  batch.seg[0] = Segment{dst, nullptr, a, b, n};
+  return LaunchSegments(batch, dtype, DefaultTuning(), stream);
+}
+
+hipError_t LaunchCopy(void* dst, const void* a, size_t n, int dtype, hipStream_t stream) {
+  SegmentBatch batch;
+  batch.count = 1;
+  batch.seg[0] = Segment{dst, nullptr, a, nullptr, n};
+  return LaunchSegments(batch, dtype, DefaultTuning(), stream);
+}
+
+}  // namespace ibcomm_hip

@@ -1,0 +1,78 @@
+// Cooperative driver: one host thread steps every emulated rank of a loopback world.
+//
+// The reference runs one process per rank and lets each spin in its own polling loop.  With all
+// ranks on one GPU a single thread can do the same job deterministically: call Progress() on each
+// rank in turn until all have issued their whole plan.  Progress() never waits, so a full sweep in
+// which no rank moved means the plans do not fit together; that is reported instead of spinning.
+#pragma once
+
+#include <vector>
+
+#include "engine.hpp"
+
+namespace ibcomm_hip {
+
+// Issues one allreduce on every rank.  With `synchronize` the call returns when all results are in
+// place (the reference's blocking semantics); without it only the host-side issue is done and the
+// caller synchronises (used while recording a graph).
+template <class B>
+int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const void* const* sendbufs,
+             void* const* recvbufs, size_t len_elements, bool synchronize) {
+  if (n < 1) return Fail(kInvalidArgument, "empty world");
+  for (int r = 0; r < n; r++) {
+    if (comms[r]->world_size() != n || comms[r]->rank() != r)
+      return Fail(kInvalidArgument, "communicator %d is rank %d of %d, expected rank %d of %d", r, comms[r]->rank(),
+                  comms[r]->world_size(), r, n);
+  }
+  int rc = kOk;
+  int begun = 0;
+  for (; begun < n; begun++) {
+    rc = comms[begun]->Begin(algo, dtype, sendbufs[begun], recvbufs[begun], len_elements);
+    if (rc != kOk) break;
+  }
+  if (rc == kOk) {
+    std::vector<char> done(n, 0);
+    int remaining = n;
+    while (remaining > 0 && rc == kOk) {
+      bool any = false;
+      for (int r = 0; r < n && rc == kOk; r++) {
+        if (done[r]) continue;
+        bool progressed = false, finished = false;
+        rc = comms[r]->Progress(&progressed, &finished);
+        any = any || progressed || finished;
+        if (finished) {
+          done[r] = 1;
+          remaining--;
+        }
+      }
+      if (rc == kOk && remaining > 0 && !any) {
+        int stuck = 0;
+        while (done[stuck]) stuck++;
+        rc = Fail(kTransportError, "loopback world made no progress: rank %d stopped at receive %zu/%zu, send %zu/%zu", stuck,
+                  comms[stuck]->recv_cursor(), comms[stuck]->recv_total(), comms[stuck]->send_cursor(),
+                  comms[stuck]->send_total());
+      }
+    }
+  }
+  if (rc != kOk) {
+    // keep the message of the first failure
+    char saved[512];
+    strncpy(saved, LastErrorBuffer(), sizeof saved);
+    saved[sizeof saved - 1] = 0;
+    for (int r = 0; r < begun; r++) comms[r]->Abort();
+    comms[0]->fabric()->Reset();
+    strncpy(LastErrorBuffer(), saved, 512);
+    return rc;
+  }
+  for (int r = 0; r < n; r++) {
+    if (synchronize) {
+      const int f = comms[r]->Finish(false);  // every rank's streams are drained below or here
+      if (f != kOk && rc == kOk) rc = f;
+    } else {
+      comms[r]->FinishNoSync();
+    }
+  }
+  return rc;
+}
+
+}  // namespace ibcomm_hip

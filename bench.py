@@ -1,0 +1,289 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X allreduce hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
+
+One "step" is one complete emulated allreduce: all N emulated ranks of the chosen BASELINE
+configuration run their whole chunk schedule on the one GPU (sendbufs resident in HBM before the
+timed region starts; every rank's recvbuf is produced).  The headline `value` is the allreduce
+algorithm bandwidth of that emulated schedule, len * 4 B / time per step, with the N ranks
+time-sharing the GPU; `extra.rank_share_algbw_GBps` is N times that (one rank's 1/N share of the
+device work).  Default workload: configs[1] of BASELINE.json (ring, 8 ranks, 256 MiB fp32 per rank,
+IBCOMM_CHUNKSIZE = 8 MiB).
+
+Two more legs, both on rank 0 of a one-GPU run:
+  roofline      the dominant kernel (the segment reduction, dst = a + b at 12 B per fp32 element)
+                launched at the shape the schedule launches it, back to back on one stream, timed
+                with HIP events recorded on that stream.
+  cpu_baseline  the CPU oracle's restatement of the reference's AllreduceRing<float> (scalar loop,
+                gcc -O2, one thread per emulated rank) on the same workload, timed on the host.
+The oracle is used only as that baseline and as the checker of the final result.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+
+CONFIGS = {
+    # id: (algo name, ranks, elements per rank, IBCOMM_CHUNKSIZE, data)
+    2: ("ring", 8, 67108864, 8388608, "normal"),
+    3: ("rabenseifner", 16, 102760448, 4194304, "normal1e-2"),
+    4: ("ring", 8, 16777216, 65536, "uniform"),
+    5: ("ring", 32, 536870911, 16777216, "normal"),
+}
+
+
+def make_inputs(torch, world, n, kind, seed):
+    out = []
+    for r in range(world):
+        g = torch.Generator(device="cuda").manual_seed(seed + r)
+        if kind == "normal":
+            t = torch.randn(n, device="cuda", generator=g)
+        elif kind == "normal1e-2":
+            t = torch.randn(n, device="cuda", generator=g) * 1e-2
+        else:
+            t = torch.rand(n, device="cuda", generator=g) * 2 - 1
+        out.append(t)
+    return out
+
+
+def check_result(torch, O, H, algo, send, recv, chunk):
+    """Bit-exact check of the last step's result: every rank on one chunk group with torch's fp32 adds
+    in the reference's order, and rank 0's first and last chunk against the oracle on the host."""
+    import numpy as np
+    world, n = len(send), send[0].numel()
+    rc, ranges = O.split_buffer(n, 4, world, chunk)
+    assert rc == 0
+    groups = O.rank_to_chunk(len(ranges), world)
+    it = torch.int32
+    if algo == H.RING:
+        g = world // 2
+        s, e = ranges[groups[g][0]][0], ranges[groups[g][-1]][1]
+        acc = send[g][s:e].clone()
+        for j in range(1, world):
+            acc += send[(g + j) % world][s:e]
+    else:
+        s, e = ranges[groups[0][0]][0], ranges[groups[0][-1]][1]
+        level = [t[s:e] for t in send]
+        while len(level) > 1:
+            level = [level[i] + level[i + 1] for i in range(0, len(level), 2)]
+        acc = level[0]
+    ok = all(torch.equal(recv[r][s:e].view(it), acc.view(it)) for r in range(world))
+    owner = {c: gi for gi, cs in enumerate(groups) for c in cs}
+    for c in (0, len(ranges) - 1):
+        s, e = ranges[c]
+        host = [t[s:e].cpu().numpy() for t in send]
+        if algo == H.RING:
+            rot = host[owner[c]:] + host[:owner[c]]
+            want = rot[0].copy()
+            for x in rot[1:]:
+                O.lib().orc_reduce_inplace(O.F32, want.ctypes.data, x.ctypes.data, want.size)
+        else:
+            rc, want = O.closed_form_tree(host)
+        ok = ok and np.array_equal(recv[0][s:e].cpu().numpy().view(np.uint32), want.view(np.uint32))
+    return bool(ok)
+
+
+def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
+    """Average duration of the dominant kernel at its in-schedule launch shape, HIP events on its own stream."""
+    world = len(send)
+    stream = torch.cuda.Stream()
+    k = segs_per_launch
+    vp = C.c_void_p
+    n = send[0].numel()
+    per_buf = max(1, n // seg_elems)
+    # rotate through the ranks' buffers so that successive launches touch different memory
+    shapes = []
+    for i in range(world * 2):
+        dst, a, b = [], [], []
+        for j in range(k):
+            idx = (i * k + j)
+            r = idx % world
+            off = ((idx // world) % per_buf) * seg_elems * 4
+            dst.append(recv[r].data_ptr() + off)
+            a.append(send[r].data_ptr() + off)
+            b.append(send[(r + 1) % world].data_ptr() + off)
+        shapes.append(((vp * k)(*dst), (vp * k)(*a), (vp * k)(*b), (C.c_size_t * k)(*([seg_elems] * k))))
+    L = H.lib()
+
+    def launch(i):
+        d, a, b, ln = shapes[i % len(shapes)]
+        rc = L.ibcomm_hip_reduce_segments(H.F32, k, d, a, b, ln, stream.cuda_stream)
+        assert rc == 0, H.last_error()
+
+    with torch.cuda.stream(stream):
+        for i in range(5):
+            launch(i)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(launches):
+            launch(i)
+        e1.record(stream)
+    e1.synchronize()
+    avg_s = e0.elapsed_time(e1) * 1e-3 / launches
+    algorithmic = 12.0 * seg_elems * k
+    return {
+        "bound": "hbm",
+        "achieved": round(algorithmic / avg_s * 1e-9, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "kernel": "ibcomm_hip::SegmentKernel<float, f32x4, 256, 1, true>",
+        "launch_shape": "%d segments x %d fp32" % (k, seg_elems),
+        "algorithmic_bytes_per_launch": int(algorithmic),
+        "avg_launch_us": round(avg_s * 1e6, 2),
+        "launches_timed": launches,
+    }
+
+
+def cpu_baseline_leg(O, world, n, chunk, algo_name):
+    """The oracle's CPU ring (AllreduceRing<float> restated) on the same workload, one thread per rank."""
+    import numpy as np
+    bufs = [np.random.default_rng(900 + r).standard_normal(n).astype(np.float32) for r in range(world)]
+    algo = O.RING_CPU if algo_name == "ring" else O.RABEN_CPU
+    times = []
+    for i in range(3):  # 1 warm-up + 2 timed
+        t0 = time.perf_counter()
+        rc, recv, _ = O.allreduce(algo, bufs, chunk if algo_name == "ring" else None)
+        t1 = time.perf_counter()
+        assert rc == 0
+        if i:
+            times.append(t1 - t0)
+        del recv
+    t = min(times)
+    single = O.lib().orc_time_reduce_f32(16 * 1024 * 1024, 5)
+    return {
+        "value": round(n * 4 / t * 1e-9, 3),
+        "unit": "GB/s algbw",
+        "cores": min(world, os.cpu_count() or 1),
+        "kind": "port",
+        "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 2 after 1 warm-up, "
+                  "one host thread per emulated rank on %d logical CPUs" % (algo_name, world, n, chunk, os.cpu_count() or 1),
+        "seconds": round(t, 3),
+        "single_core_reduce_loop_GBps": round(12.0 * 16 * 1024 * 1024 / single * 1e-9, 2),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
+    ap.add_argument("--landing", choices=["memcpy", "kernel", "direct"], default=None)
+    ap.add_argument("--fuse", type=int, default=None)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: every emulated rank lives on the same MI355X and nothing in this build "
+              "uses a second device; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py is a single-process, single-GPU benchmark; do not launch it under torchrun", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import hip_lib as H
+    import oracle_lib as O
+
+    algo_name, world, n, chunk, kind = CONFIGS[args.config]
+    algo = H.RING if algo_name == "ring" else H.RABENSEIFNER
+    torch.cuda.set_device(0)
+    os.environ["IBCOMM_CHUNKSIZE"] = str(chunk)
+    if args.config == 4:
+        os.environ.setdefault("IBCOMM_NUM_CUDA_STREAM", "64")
+
+    send = make_inputs(torch, world, n, kind, 1234)
+    recv = [torch.empty_like(t) for t in send]
+    sp = [t.data_ptr() for t in send]
+    rp = [t.data_ptr() for t in recv]
+
+    with H.World(world) as w:
+        if args.landing:
+            w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT}[args.landing])
+        if args.fuse:
+            w.set_max_fuse(args.fuse)
+        for _ in range(args.warmup):
+            assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0, H.last_error()
+        torch.cuda.synchronize()
+        w.reset_stats()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            rc = w.allreduce_ptrs(algo, H.F32, sp, rp, n)
+            assert rc == 0, H.last_error()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        st = [w.stats(r) for r in range(world)]
+
+    sec_per_step = (t1 - t0) / args.steps
+    parity = check_result(torch, O, H, algo, send, recv, chunk)
+
+    steps = args.steps
+    total = {k: sum(s[k] for s in st) for k in st[0]}
+    device_bytes_per_step = (12 * total["reduce_elements"] + 2 * total["landing_bytes"] + 2 * total["gather_bytes"]) / steps
+    segs_per_launch = max(1, round(st[0]["reduce_segments"] / max(1, st[0]["reduce_launches"])))
+    seg_elems = st[0]["reduce_elements"] // max(1, st[0]["reduce_segments"])
+
+    algbw = n * 4 / sec_per_step * 1e-9
+    line = {
+        "metric": "emulated allreduce algbw (GB/s) with reduce-kernel HBM roofline, fp32",
+        "value": round(algbw, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[%d]: %s allreduce, %d emulated ranks on one GPU, %d fp32 (%.0f MiB) per rank, "
+                        "IBCOMM_CHUNKSIZE=%d, all ranks' schedules executed per step" % (
+                            args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk),
+            "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk,
+            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "memcpy"),
+            "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "48")),
+        },
+        "parity_bit_exact": parity,
+        "extra": {
+            "busbw_GBps": round(algbw * 2 * (world - 1) / world, 2),
+            "rank_share_algbw_GBps": round(algbw * world, 2),
+            "device_traffic_GB_per_step": round(device_bytes_per_step * 1e-9, 3),
+            "aggregate_device_GBps": round(device_bytes_per_step / sec_per_step * 1e-9, 1),
+            "aggregate_frac_of_hbm_peak": round(device_bytes_per_step / sec_per_step * 1e-9 / HBM_PEAK_GBPS, 4),
+            "rank0_reduce_launches_per_step": st[0]["reduce_launches"] / steps,
+            "rank0_segments_per_launch": segs_per_launch,
+            "rank0_reduce_elements_per_step": st[0]["reduce_elements"] // steps,
+            "rank0_landing_copies_per_step": st[0]["landing_copies"] / steps,
+            "rank0_gather_copies_per_step": st[0]["gather_copies"] / steps,
+            "streams_per_rank": st[0]["streams_created"],
+            "pool_slots_high_water": max(s["slots_high_water"] for s in st),
+        },
+    }
+    if not args.no_roofline:
+        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, 200)
+    del recv
+    if not args.no_cpu:
+        del send
+        torch.cuda.empty_cache()
+        line["cpu_baseline"] = cpu_baseline_leg(O, world, n, chunk, algo_name)
+    print(json.dumps(line))
+    if not parity:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,175 @@
+/*
+ * C ABI of the MI355X allreduce hot path (libibcomm_hip.so).
+ *
+ * This is the boundary a binding of PFNProto's IBVerbsCommunicator would call
+ * for the device allreduce path.  The reference exposes that path as C++
+ * member templates instantiated in the caller's translation unit
+ * (ibcomm/ibverbs_communicator.h:101-115, bodies in
+ * ibcomm/allreduce_cuda_impl.h); there is no exported symbol per element type.
+ * Each entry point below names the reference interface it stands for.
+ *
+ * Conventions
+ *   - Plain pointers and sizes only.  Buffers passed to the allreduce and
+ *     reduce calls are DEVICE pointers on the current HIP device.
+ *   - Every function returns 0 on success or one of the reference's exit codes
+ *     (ibcomm/util.h:32-42): 1 invalid argument, 2 transport error, 3 HIP
+ *     error, 4 not supported.  Where the reference prints a message and calls
+ *     exit(code) (util.h:44-52) this library returns the code and keeps the
+ *     message for ibcomm_hip_last_error(); the C++ facade
+ *     (allreduce-proto_amd/ibcomm/ibverbs_communicator.h) prints and exits.
+ *   - The network is an in-process loopback: all ranks of a world live in one
+ *     process on one GPU and exchange chunks through device memory.
+ *   - Environment knobs keep the reference's names: IBCOMM_CHUNKSIZE (read on
+ *     every allreduce), IBCOMM_NUM_CUDA_STREAM, IBCOMM_MEMORY_POOL_PRE_ALLOC,
+ *     IBCOMM_WORK_GPU_MEMORY_SIZE (read when a communicator is created).
+ */
+#ifndef IBCOMM_HIP_H_
+#define IBCOMM_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ibcomm_hip_fabric ibcomm_hip_fabric; /* the loopback "network" of one world */
+typedef struct ibcomm_hip_comm ibcomm_hip_comm;     /* one rank's IBVerbsCommunicator */
+typedef struct ibcomm_hip_plan ibcomm_hip_plan;     /* read-only view of one rank's message plan */
+
+/* ibcomm/util.h:32-42 */
+enum {
+  IBCOMM_HIP_OK = 0,
+  IBCOMM_HIP_INVALID_ARGUMENT = 1,
+  IBCOMM_HIP_TRANSPORT_ERROR = 2, /* IBVERBS_ERROR */
+  IBCOMM_HIP_DEVICE_ERROR = 3,    /* CUDA_ERROR */
+  IBCOMM_HIP_NOT_SUPPORTED = 4
+};
+
+/* element types the templates are instantiated with: float (examples/allreduce.cpp:103-111),
+ * int (ibcomm/allreduce_tester.cpp:416); double and 64-bit integers come for free */
+enum { IBCOMM_HIP_F32 = 0, IBCOMM_HIP_I32 = 1, IBCOMM_HIP_F64 = 2, IBCOMM_HIP_I64 = 3 };
+
+enum { IBCOMM_HIP_RING = 0, IBCOMM_HIP_RABENSEIFNER = 1 };
+
+/* Message of the last failure on the calling thread (what util::IbcommError would have printed). */
+const char* ibcomm_hip_last_error(void);
+
+/* ---- bring-up ----------------------------------------------------------------------------- */
+
+/* Stands for the queue-pair wiring the reference does with CreateQueuePair / RegisterQueuePair
+ * and an out-of-band MPI_Alltoall (examples/allreduce.cpp:50-77): creates the channels between
+ * world_size emulated ranks. */
+int ibcomm_hip_fabric_create(int world_size, ibcomm_hip_fabric** out);
+int ibcomm_hip_fabric_destroy(ibcomm_hip_fabric* fabric);
+
+/* IBVerbsCommunicator::IBVerbsCommunicator(int world_size) + Init + PrepareMemoryPool
+ * (ibcomm/ibverbs_communicator.cpp:24-99, ibcomm/ibverbs_communicator_cuda.cpp:26-37):
+ * allocates the HBM staging pool and reads the pool knobs. */
+int ibcomm_hip_comm_create(ibcomm_hip_fabric* fabric, int world_size, ibcomm_hip_comm** out);
+/* IBVerbsCommunicator::~IBVerbsCommunicator (ibcomm/ibverbs_communicator.cpp:101-155) */
+int ibcomm_hip_comm_destroy(ibcomm_hip_comm* comm);
+/* IBVerbsCommunicator::RegisterMyself (ibcomm/ibverbs_communicator.cpp:355-357) */
+int ibcomm_hip_comm_register_myself(ibcomm_hip_comm* comm, int my_rank);
+
+/* ---- the hot path ------------------------------------------------------------------------- */
+
+/* IBVerbsCommunicator::AllreduceRingCuda<T>(const T* sendbuf, T* recvbuf, size_t len_elements)
+ * (ibcomm/allreduce_cuda_impl.h:35-301).  Blocking; every rank of the world must be inside the
+ * same call on a thread of its own, as every process is in the reference.  On return recvbuf
+ * holds, for each element, the left fold of the ranks' values starting at the rank that owns the
+ * element's chunk group. */
+int ibcomm_hip_allreduce_ring(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
+                              size_t len_elements);
+/* IBVerbsCommunicator::AllreduceRabenseifnerCuda<T> (ibcomm/allreduce_cuda_impl.h:326-717).
+ * Power-of-two worlds only (returns 4 otherwise); the result is the balanced pairwise tree over
+ * rank index. */
+int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
+                                      size_t len_elements);
+
+/* Typed spellings of the two calls above, one per template instantiation the reference's own
+ * programs use. */
+int ibcomm_hip_allreduce_ring_f32(ibcomm_hip_comm* comm, const float* sendbuf, float* recvbuf, size_t len_elements);
+int ibcomm_hip_allreduce_ring_i32(ibcomm_hip_comm* comm, const int32_t* sendbuf, int32_t* recvbuf, size_t len_elements);
+int ibcomm_hip_allreduce_rabenseifner_f32(ibcomm_hip_comm* comm, const float* sendbuf, float* recvbuf,
+                                          size_t len_elements);
+int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* comm, const int32_t* sendbuf, int32_t* recvbuf,
+                                          size_t len_elements);
+
+/* The same collectives for a whole loopback world driven from ONE host thread: comms[r],
+ * sendbufs[r], recvbufs[r] belong to rank r, r = 0 .. world_size-1.  Equivalent to world_size
+ * concurrent calls of the per-rank functions (which is how mpiexec runs the reference,
+ * tests/allreduce_test.py:91), without needing the threads. */
+int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
+                               const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
+
+/* The reduction kernel on its own, asynchronous on `stream` (a hipStream_t, NULL = default
+ * stream): dst[i] = a[i] + b[i].  Stands for _reduce_inplace_cuda<T>
+ * (ibcomm/allreduce_cuda_impl.h:26-33, launches at :132-133 and :510-512), which is the case
+ * dst == a. */
+int ibcomm_hip_reduce(int dtype, void* dst, const void* a, const void* b, size_t len_elements, void* stream);
+/* Several independent segments in one launch (at most ibcomm_hip_max_segments()). */
+int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, const void* const* a,
+                               const void* const* b, const size_t* len_elements, void* stream);
+int ibcomm_hip_max_segments(void);
+
+/* ---- partitioning and plans (host only, no device needed) ---------------------------------- */
+
+/* IBVerbsCommunicator::SplitBuffer (ibcomm/ibverbs_communicator.cpp:637-683).  env_chunksize is
+ * the text IBCOMM_CHUNKSIZE would hold, NULL for "unset".  Writes up to cap ranges
+ * [starts[i], ends[i]) and the total count to *n_ranges. */
+int ibcomm_hip_split_buffer(size_t len_elements, size_t sizeof_element, int world_size, const char* env_chunksize,
+                            size_t* starts, size_t* ends, int cap, int* n_ranges);
+/* IBVerbsCommunicator::GetRankToChunk (ibcomm/ibverbs_communicator.cpp:685-707): rank r owns
+ * chunks first_chunk[r] .. first_chunk[r] + n_chunks[r] - 1. */
+int ibcomm_hip_rank_to_chunk(int n_ranges, int world_size, int* first_chunk, int* n_chunks);
+/* util::GetExpOfTwo (ibcomm/util.h:156-175) */
+int ibcomm_hip_get_exp_of_two(int n);
+
+/* The ordered messages one rank consumes and emits: the content of the reference's reg_q /
+ * first_send_q (ibcomm/allreduce_cuda_impl.h:61-89) and recv_q / send_q / first_send_q
+ * (:387-466).  kind: 0 = add to sendbuf's chunk, 1 = add to the running sum, 2 = store. */
+int ibcomm_hip_plan_create(int algo, int world_size, int rank, size_t len_elements, size_t sizeof_element,
+                           const char* env_chunksize, ibcomm_hip_plan** out);
+void ibcomm_hip_plan_destroy(ibcomm_hip_plan* plan);
+int ibcomm_hip_plan_counts(const ibcomm_hip_plan* plan, int* n_chunks, int* n_recvs, int* n_sends);
+int ibcomm_hip_plan_range(const ibcomm_hip_plan* plan, int chunk, size_t* begin, size_t* end);
+int ibcomm_hip_plan_recv(const ibcomm_hip_plan* plan, int k, int* chunk, int* peer, int* kind);
+int ibcomm_hip_plan_send(const ibcomm_hip_plan* plan, int k, int* chunk, int* peer, int* dep);
+
+/* ---- knobs and counters --------------------------------------------------------------------- */
+
+/* Chunks reduced per kernel launch at most (1 = one launch per chunk, like the reference). */
+int ibcomm_hip_comm_set_max_fuse(ibcomm_hip_comm* comm, int max_chunks_per_launch);
+/* How a message reaches the reduction: 0 = hipMemcpyAsync into a pool slot, 1 = one copy-kernel
+ * launch for all messages of a pass, 2 = the reduction reads the sender's buffer directly. */
+int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode);
+
+typedef struct {
+  uint64_t calls;
+  uint64_t reduce_launches;
+  uint64_t reduce_segments;
+  uint64_t reduce_elements;
+  uint64_t landing_copies;
+  uint64_t landing_bytes;
+  uint64_t gather_copies;
+  uint64_t gather_bytes;
+  uint64_t messages_sent;
+  uint64_t messages_received;
+  uint64_t events_recorded;
+  uint64_t stream_waits;
+  uint64_t streams_created;
+  uint64_t slots_high_water;
+  uint64_t slot_count;
+  uint64_t pool_blocks;
+  uint64_t pool_bytes;
+  uint64_t progress_passes;
+} ibcomm_hip_stats;
+
+int ibcomm_hip_comm_stats(ibcomm_hip_comm* comm, ibcomm_hip_stats* out);
+int ibcomm_hip_comm_reset_stats(ibcomm_hip_comm* comm);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IBCOMM_HIP_H_ */

@@ -1,0 +1,79 @@
+"""ctypes view of tests/support/libibcomm_sim.so: the allreduce engine on a simulated device.
+
+Test infrastructure.  The simulated device records streams/events/copies/launches as a dependency
+graph, runs it in random topological order and checks it for unordered conflicting accesses; it
+exists so that the engine's host logic is tested on the CPU.  It is not part of the product.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SIM_SO = os.path.join(HERE, "support", "libibcomm_sim.so")
+
+
+class EngineStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "calls", "reduce_launches", "reduce_segments", "reduce_elements", "landing_copies", "landing_bytes",
+        "gather_copies", "gather_bytes", "messages_sent", "messages_received", "events_recorded", "stream_waits",
+        "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes")]
+
+
+class Report(C.Structure):
+    _fields_ = [("rc", C.c_int), ("nodes", C.c_long), ("races", C.c_long), ("unrecorded_waits", C.c_long),
+                ("rank0", EngineStats), ("error", C.c_char * 512), ("first_race", C.c_char * 256)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        subprocess.check_call(["make", "-s", "-C", os.path.join(HERE, "support")])
+        _lib = C.CDLL(SIM_SO)
+        _lib.sim_world_allreduce.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                             C.c_size_t, C.c_int, C.c_int, C.c_uint, C.c_int, C.c_int, C.POINTER(Report)]
+    return _lib
+
+
+DT = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.float64): 2, np.dtype(np.int64): 3}
+
+
+def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, threaded=False, repeats=1,
+              pool_bytes=1 << 16, in_place=False, streams=None):
+    """-> (rc, [recvbuf per rank], Report).  Environment knobs are set for the duration of the call."""
+    world = len(sendbufs)
+    sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]
+    n = sendbufs[0].size
+    if in_place:
+        recv = sendbufs
+    else:
+        recv = []
+        for _ in range(world):
+            r = np.empty(n, dtype=sendbufs[0].dtype)
+            r.view(np.uint8)[:] = 0x55
+            recv.append(r)
+    sp = (C.c_void_p * world)(*[s.ctypes.data for s in sendbufs])
+    rp = (C.c_void_p * world)(*[r.ctypes.data for r in recv])
+    saved = {k: os.environ.get(k) for k in ("IBCOMM_CHUNKSIZE", "IBCOMM_MEMORY_POOL_PRE_ALLOC", "IBCOMM_NUM_CUDA_STREAM")}
+    try:
+        if chunksize is None:
+            os.environ.pop("IBCOMM_CHUNKSIZE", None)
+        else:
+            os.environ["IBCOMM_CHUNKSIZE"] = str(chunksize)
+        os.environ["IBCOMM_MEMORY_POOL_PRE_ALLOC"] = str(pool_bytes)
+        if streams is not None:
+            os.environ["IBCOMM_NUM_CUDA_STREAM"] = str(streams)
+        rep = Report()
+        rc = lib().sim_world_allreduce(algo, DT[sendbufs[0].dtype], world, sp, rp, n, max_fuse, landing, seed,
+                                       1 if threaded else 0, repeats, C.byref(rep))
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    return rc, recv, rep

@@ -1,0 +1,80 @@
+// C entry points that run the allreduce engine on the simulated device (see sim_backend.hpp).
+// TEST INFRASTRUCTURE ONLY.
+#include <memory>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "sim_backend.hpp"
+#include "engine.hpp"
+#include "world.hpp"
+
+using namespace ibcomm_hip;
+using ibcomm_sim::Sim;
+using ibcomm_sim::SimBackend;
+
+extern "C" {
+
+struct sim_report {
+  int rc;
+  long nodes;
+  long races;             // -1: graph too large to check
+  long unrecorded_waits;
+  EngineStats rank0;
+  char error[512];
+  char first_race[256];
+};
+
+// threaded = 0: one thread steps all ranks (RunWorld); 1: one thread per rank (AllreduceBlocking).
+// repeats > 1 runs the same collective again on the same communicators (event/slot reuse).
+int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,
+                        int max_fuse, int landing, unsigned seed, int threaded, int repeats, sim_report* rep) {
+  *rep = sim_report();
+  Sim::Get().Reset(seed);
+  Fabric<SimBackend> fabric(world);
+  std::vector<std::unique_ptr<Communicator<SimBackend>>> comms;
+  std::vector<Communicator<SimBackend>*> raw;
+  int rc = kOk;
+  for (int r = 0; r < world && rc == kOk; r++) {
+    comms.emplace_back(new Communicator<SimBackend>(&fabric, world));
+    rc = comms.back()->Init();
+    comms.back()->RegisterMyself(r);
+    comms.back()->set_max_fuse(max_fuse);
+    comms.back()->set_landing(landing);
+    raw.push_back(comms.back().get());
+  }
+  for (int k = 0; k < repeats && rc == kOk; k++) {
+    if (!threaded) {
+      rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, true);
+      if (rc != kOk) snprintf(rep->error, sizeof rep->error, "%s", LastErrorBuffer());
+    } else {
+      std::vector<int> rcs(world, 0);
+      std::vector<std::string> msgs(world);
+      std::vector<std::thread> th;
+      for (int r = 0; r < world; r++) {
+        th.emplace_back([&, r]() {
+          rcs[r] = raw[r]->AllreduceBlocking(algo, dtype, sendbufs[r], recvbufs[r], len);
+          if (rcs[r]) msgs[r] = LastErrorBuffer();
+        });
+      }
+      for (auto& t : th) t.join();
+      for (int r = 0; r < world; r++) {
+        if (rcs[r] && rc == kOk) {
+          rc = rcs[r];
+          snprintf(rep->error, sizeof rep->error, "%s", msgs[r].c_str());
+        }
+      }
+    }
+  }
+  if (rc != kOk && !rep->error[0]) snprintf(rep->error, sizeof rep->error, "%s", LastErrorBuffer());
+  std::string first;
+  rep->rc = rc;
+  rep->nodes = Sim::Get().node_count();
+  rep->races = threaded ? -1 : Sim::Get().CheckRaces(&first);
+  rep->unrecorded_waits = Sim::Get().unrecorded_waits();
+  if (!raw.empty()) rep->rank0 = raw[0]->stats();
+  snprintf(rep->first_race, sizeof rep->first_race, "%s", first.c_str());
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,152 @@
+"""Host-logic tests of the allreduce engine (allreduce-proto_amd/csrc/engine.hpp, plan.hpp, loopback.hpp,
+memory_pool.hpp) on a simulated device.
+
+The same engine templates the product instantiates with the HIP runtime are instantiated here with
+tests/support/sim_backend.hpp, which defers every copy and launch, runs them in a random order that
+respects the recorded stream/event dependencies, and checks that every pair of conflicting memory
+accesses is ordered.  Results must be bit-identical to the oracle's restatement of
+AllreduceRingCuda / AllreduceRabenseifnerCuda.
+"""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import sim_lib as S
+
+RING, RABEN = 0, 1
+ORACLE_ALGO = {RING: O.RING_GPU, RABEN: O.RABEN_GPU}
+
+
+def rand_bufs(world, n, seed=0, dtype=np.float32):
+    return [(np.random.default_rng(seed + r).standard_normal(n) * 3).astype(dtype) for r in range(world)]
+
+
+def check(algo, bufs, chunk=None, **kw):
+    rc, recv, rep = S.allreduce(algo, bufs, chunk, **kw)
+    assert rc == 0, rep.error.decode()
+    orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs, chunk)
+    assert orc == 0
+    for r in range(len(bufs)):
+        assert np.array_equal(O.bits(recv[r]), O.bits(want[r])), "rank %d differs from the oracle" % r
+    assert rep.unrecorded_waits == 0
+    if not kw.get("threaded"):
+        assert rep.races == 0, rep.first_race.decode()
+    return rep
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("fuse", [1, 3, 48])
+@pytest.mark.parametrize("world", [2, 3, 4, 5, 8])
+def test_ring_matches_oracle(world, fuse, landing):
+    for n, chunk in [(world, None), (4 * world + 1, None), (1000 + world, None), (512, 16)]:
+        if chunk and -(-n // (chunk // 4)) < 2 * world:
+            continue
+        check(RING, rand_bufs(world, n, seed=n), chunk, max_fuse=fuse, landing=landing, seed=world * 7 + fuse)
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("fuse", [1, 3, 48])
+@pytest.mark.parametrize("world", [2, 4, 8, 16])
+def test_rabenseifner_matches_oracle(world, fuse, landing):
+    for n, chunk in [(world, None), (4 * world + 3, None), (2000 + world, None), (1024, 16)]:
+        if chunk and -(-n // (chunk // 4)) < 2 * world:
+            continue
+        check(RABEN, rand_bufs(world, n, seed=n + 1), chunk, max_fuse=fuse, landing=landing, seed=world * 11 + fuse)
+
+
+@pytest.mark.parametrize("algo,world", [(RING, 4), (RING, 3), (RABEN, 4), (RABEN, 8)])
+def test_many_random_schedules(algo, world):
+    bufs = rand_bufs(world, 777, seed=42)
+    for seed in range(12):
+        check(algo, bufs, 32, max_fuse=1 + seed % 5, landing=seed % 3, seed=seed, streams=1 + seed % 4)
+
+
+@pytest.mark.parametrize("algo,world", [(RING, 4), (RABEN, 4)])
+def test_tiny_pool_forces_slot_reuse(algo, world):
+    # two slots only: every landing has to order itself after the previous reader of its slot
+    bufs = rand_bufs(world, 4096, seed=3)
+    stride = 256 + 256  # 64-byte chunks + 16 B margin round up to 256; pool of 512 B gives two slots
+    for fuse in (1, 2, 7):
+        rep = check(algo, bufs, 64, max_fuse=fuse, landing=0, pool_bytes=stride, seed=fuse)
+        assert rep.rank0.slot_count >= 2
+    # a pool smaller than one chunk grows instead of failing
+    rep = check(algo, bufs, 1024, max_fuse=4, landing=1, pool_bytes=64, seed=9)
+    assert rep.rank0.pool_blocks >= 2
+
+
+@pytest.mark.parametrize("algo,world", [(RING, 2), (RING, 4), (RABEN, 2), (RABEN, 8)])
+def test_threads_one_per_rank(algo, world):
+    bufs = rand_bufs(world, 3000, seed=8)
+    for rep_i in range(3):
+        check(algo, bufs, 64, max_fuse=4, landing=rep_i % 3, threaded=True, seed=rep_i)
+
+
+@pytest.mark.parametrize("algo", [RING, RABEN])
+def test_repeated_calls_reuse_events_and_slots(algo):
+    bufs = rand_bufs(4, 2048, seed=5)
+    rep = check(algo, bufs, 64, max_fuse=3, repeats=4, seed=1)
+    assert rep.rank0.calls == 4
+    check(algo, bufs, 64, max_fuse=3, repeats=3, threaded=True, seed=2)
+
+
+@pytest.mark.parametrize("algo,world", [(RING, 3), (RING, 4), (RABEN, 4)])
+def test_in_place(algo, world):
+    bufs = rand_bufs(world, 1500, seed=6)
+    orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs)
+    for landing in (0, 1, 2):
+        rc, recv, rep = S.allreduce(algo, bufs, max_fuse=5, landing=landing, in_place=True, seed=landing)
+        assert rc == 0, rep.error.decode()
+        for r in range(world):
+            assert np.array_equal(O.bits(recv[r]), O.bits(want[r]))
+        assert rep.races == 0, rep.first_race.decode()
+
+
+def test_single_rank_is_a_copy():
+    bufs = rand_bufs(1, 100)
+    for algo in (RING, RABEN):
+        rc, recv, rep = S.allreduce(algo, bufs)
+        assert rc == 0 and np.array_equal(O.bits(recv[0]), O.bits(bufs[0]))
+
+
+def test_dtypes():
+    for dtype in (np.int32, np.float64, np.int64):
+        bufs = [(np.random.default_rng(r).standard_normal(500) * 1000).astype(dtype) for r in range(4)]
+        check(RING, bufs, max_fuse=4)
+        check(RABEN, bufs, max_fuse=4)
+
+
+def test_error_codes_match_reference():
+    # tests/allreduce_test.py:198-225 and :132-153
+    bufs = [np.arange(256, dtype=np.int32) for _ in range(4)]
+    for chunk in ["0", "1", "2", "3", "-128", "1k", "1024"]:
+        rc, _, rep = S.allreduce(RING, bufs, chunk)
+        assert rc == 1, (chunk, rep.error)
+    one = [np.ones(1, dtype=np.int32) for _ in range(2)]
+    assert S.allreduce(RING, one)[0] == 4
+    assert S.allreduce(RABEN, one)[0] == 4
+    for world in (3, 5, 6):
+        assert S.allreduce(RABEN, [np.arange(2 * world, dtype=np.int32) for _ in range(world)])[0] == 4
+    # a failed call leaves the communicators usable
+    rc, recv, rep = S.allreduce(RING, bufs, "16")
+    assert rc == 0
+
+
+def test_work_per_rank_matches_the_schedule():
+    # ring, N ranks, q chunks per group: (N-1)q reductions and (N-1)q gathers per rank, 2(N-1)q messages
+    world, n, chunk = 4, 4096, 64
+    bufs = rand_bufs(world, n)
+    rep = check(RING, bufs, chunk, max_fuse=1)
+    q = n * 4 // chunk // world
+    st = rep.rank0
+    assert st.reduce_segments == (world - 1) * q and st.reduce_launches == (world - 1) * q
+    assert st.reduce_elements == (world - 1) * n // world
+    assert st.gather_bytes == (world - 1) * n // world * 4
+    assert st.messages_received == 2 * (world - 1) * q and st.messages_sent == 2 * (world - 1) * q
+    # fused: whatever has landed goes into one launch (how much that is depends on the order in
+    # which the driver visits the ranks), never more than 48 chunks
+    rep = check(RING, bufs, chunk, max_fuse=48)
+    assert -(-(world - 1) * q // 48) <= rep.rank0.reduce_launches <= world
+    assert rep.rank0.reduce_segments == (world - 1) * q
+    # Rabenseifner rank 0 of 4: halving windows of 2 and 1 groups
+    rep = check(RABEN, bufs, chunk, max_fuse=1)
+    assert rep.rank0.reduce_segments == 3 * q and rep.rank0.gather_bytes == 3 * q * chunk

@@ -1,0 +1,297 @@
+"""GPU parity of the allreduce engines through the C ABI, bit-exact against the CPU oracle's
+restatement of AllreduceRingCuda / AllreduceRabenseifnerCuda, plus the reference tester's cases
+(tests/allreduce_test.py:102-225) and the BASELINE configurations."""
+import numpy as np
+import pytest
+
+import hip_lib as H
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+import gpu_util as G  # noqa: E402
+
+
+def rand_bufs(world, n, seed=0, dtype=np.float32, scale=1.0):
+    return [(np.random.default_rng(seed + r).standard_normal(n) * scale).astype(dtype) for r in range(world)]
+
+
+def kat_bufs(world, n):
+    i = np.arange(n, dtype=np.int64)
+    return [(i * world + p).astype(np.int32) for p in range(world)]
+
+
+def kat_answer(world, n):
+    i = np.arange(n, dtype=np.int64)
+    return (i * world * world + world * (world - 1) // 2).astype(np.int32)
+
+
+# ------------------------------------------------------------------ engines vs oracle
+
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("fuse", [1, 4, 48])
+@pytest.mark.parametrize("world_size", [2, 3, 4, 8])
+def test_ring_matches_oracle(world_size, fuse, landing):
+    with H.World(world_size) as w:
+        w.set_max_fuse(fuse)
+        w.set_landing(landing)
+        for n, chunk in [(world_size, None), (4 * world_size + 1, None), (100003, None), (65536, 1024), (1 << 20, None)]:
+            G.check_against_oracle(w, H.RING, rand_bufs(world_size, n, seed=n), chunk)
+
+
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("fuse", [1, 4, 48])
+@pytest.mark.parametrize("world_size", [2, 4, 8, 16])
+def test_rabenseifner_matches_oracle(world_size, fuse, landing):
+    with H.World(world_size) as w:
+        w.set_max_fuse(fuse)
+        w.set_landing(landing)
+        for n, chunk in [(world_size, None), (4 * world_size + 3, None), (100003, None), (65536, 1024), (1 << 20, None)]:
+            G.check_against_oracle(w, H.RABENSEIFNER, rand_bufs(world_size, n, seed=n + 1, scale=1e-2), chunk)
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_one_thread_per_rank_blocking_calls(algo):
+    # the reference's usage: every rank inside its own blocking call at the same time
+    with H.World(4) as w:
+        for k in range(3):
+            G.check_against_oracle(w, algo, rand_bufs(4, 300001, seed=k), None, threads=True)
+        G.check_against_oracle(w, algo, rand_bufs(4, 65536, seed=9), 4096, threads=True)
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_repeated_calls_and_changing_shapes(algo):
+    with H.World(4) as w:
+        for k, (n, chunk) in enumerate([(50000, None), (50000, None), (777, None), (1 << 18, 16384), (50000, 1000)]):
+            G.check_against_oracle(w, algo, rand_bufs(4, n, seed=k), chunk)
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_in_place(algo):
+    with H.World(4) as w:
+        G.check_against_oracle(w, algo, rand_bufs(4, 200003, seed=2), None, in_place=True)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float64, np.int64])
+def test_element_types(dtype):
+    with H.World(4) as w:
+        bufs = [(np.random.default_rng(r).standard_normal(70001) * 1e4).astype(dtype) for r in range(4)]
+        G.check_against_oracle(w, H.RING, bufs)
+        G.check_against_oracle(w, H.RABENSEIFNER, bufs)
+
+
+def test_odd_chunk_offsets_keep_vector_path_correct():
+    # 2521 elements on 2 ranks -> chunks of 316 and a tail of 309; 1003 on 5 ranks -> chunks of 51
+    with H.World(2) as w:
+        G.check_against_oracle(w, H.RING, rand_bufs(2, 2521))
+        G.check_against_oracle(w, H.RABENSEIFNER, rand_bufs(2, 2521))
+    with H.World(5) as w:
+        G.check_against_oracle(w, H.RING, rand_bufs(5, 1003))
+
+
+# ------------------------------------------------------------------ reference tester cases
+
+def run_kat(world_size, algo, n, chunk=None):
+    with H.World(world_size) as w:
+        send = G.to_device(kat_bufs(world_size, n))
+        recv = [G.poisoned_like(t) for t in send]
+        rc = G.run_world(w, algo, send, recv, chunk)
+        return rc, [t.cpu().numpy() for t in recv]
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_1proc(algo):
+    rc, recv = run_kat(1, algo, 256)
+    assert rc == 0 and np.array_equal(recv[0], kat_bufs(1, 256)[0])
+
+
+@pytest.mark.parametrize("world_size,n", [(1, 2), (2, 4), (3, 6), (5, 10), (2, 2521)])
+def test_small_buffer_ring(world_size, n):
+    rc, recv = run_kat(world_size, H.RING, n)
+    assert rc == 0
+    for r in recv:
+        assert np.array_equal(r, kat_answer(world_size, n))
+
+
+@pytest.mark.parametrize("world_size,n,want", [(1, 2, 0), (2, 4, 0), (3, 6, 4), (5, 10, 4), (2, 2521, 0)])
+def test_small_buffer_rabenseifner(world_size, n, want):
+    rc, recv = run_kat(world_size, H.RABENSEIFNER, n)
+    assert rc == want
+    if rc == 0:
+        for r in recv:
+            assert np.array_equal(r, kat_answer(world_size, n))
+
+
+@pytest.mark.parametrize("world_size,algo", [(2, H.RING), (3, H.RING), (4, H.RING), (2, H.RABENSEIFNER), (4, H.RABENSEIFNER)])
+def test_basic_128m(world_size, algo):
+    n = 128 * 1024 * 1024 // 4
+    rc, recv = run_kat(world_size, algo, n)
+    assert rc == 0
+    want = kat_answer(world_size, n)
+    for r in recv:
+        assert np.array_equal(r, want)
+
+
+def test_basic_128m_rabenseifner_three_ranks_not_supported():
+    rc, _ = run_kat(3, H.RABENSEIFNER, 1024)
+    assert rc == H.NOT_SUPPORTED
+
+
+@pytest.mark.parametrize("chunk", [4, 8, 16, 32, 64, 128])
+def test_chunk_size(chunk):
+    rc, recv = run_kat(4, H.RING, 256, chunk)
+    assert rc == 0
+    for r in recv:
+        assert np.array_equal(r, kat_answer(4, 256))
+
+
+def test_invalid_error():
+    for chunk in ["0", "1", "2", "3", "-128", "1k"]:
+        rc, _ = run_kat(4, H.RING, 256, chunk)
+        assert rc == H.INVALID_ARGUMENT, chunk
+    with H.World(2) as w:
+        one = G.to_device([np.ones(1, dtype=np.int32)] * 2)
+        out = [G.poisoned_like(t) for t in one]
+        assert G.run_world(w, H.RING, one, out) == H.NOT_SUPPORTED
+        assert G.run_world(w, H.RABENSEIFNER, one, out) == H.NOT_SUPPORTED
+        # the world is still usable after a refused call
+        G.check_against_oracle(w, H.RING, rand_bufs(2, 1000))
+
+
+def test_aging_short():
+    # tests/allreduce_test.py:227-235 repeats 100 x 128 MiB; a short version of the same idea
+    with H.World(4) as w:
+        send = G.to_device(kat_bufs(4, 1 << 20))
+        want = torch.from_numpy(kat_answer(4, 1 << 20)).cuda()
+        for algo in (H.RING, H.RABENSEIFNER):
+            for _ in range(25):
+                recv = [G.poisoned_like(t) for t in send]
+                assert G.run_world(w, algo, send, recv) == 0
+                assert all(torch.equal(r, want) for r in recv)
+
+
+# ------------------------------------------------------------------ BASELINE configurations
+
+def device_inputs(world_size, n, seed, kind):
+    out = []
+    for r in range(world_size):
+        g = torch.Generator(device="cuda").manual_seed(seed + r)
+        if kind == "normal":
+            t = torch.randn(n, device="cuda", generator=g)
+        elif kind == "normal1e-2":
+            t = torch.randn(n, device="cuda", generator=g) * 1e-2
+        elif kind == "uniform":
+            t = torch.rand(n, device="cuda", generator=g) * 2 - 1
+        elif kind == "ints":
+            t = torch.randint(-1000, 1001, (n,), device="cuda", generator=g).float()
+        out.append(t)
+    return out
+
+
+def check_ring_on_device(send, recv, chunk):
+    world_size, n = len(send), send[0].numel()
+    rc, ranges = O.split_buffer(n, 4, world_size, chunk)
+    assert rc == 0
+    groups = O.rank_to_chunk(len(ranges), world_size)
+    for g, cids in enumerate(groups):
+        span = (ranges[cids[0]][0], ranges[cids[-1]][1])
+        want = G.device_ring_fold(send, span, g)
+        for r in range(world_size):
+            assert G.bits_equal(recv[r][span[0]:span[1]], want), "rank %d group %d" % (r, g)
+
+
+def check_stripes_against_oracle(send, recv0, algo, chunk, stripes):
+    """Sampled element ranges, recomputed on the host by the oracle's closed form."""
+    world_size, n = len(send), send[0].numel()
+    rc, ranges = O.split_buffer(n, 4, world_size, chunk)
+    groups = O.rank_to_chunk(len(ranges), world_size)
+    owner_of_chunk = {c: g for g, cids in enumerate(groups) for c in cids}
+    for c in stripes:
+        s, e = ranges[c]
+        host = [t[s:e].cpu().numpy() for t in send]
+        if algo == H.RING:
+            g = owner_of_chunk[c]
+            rot = host[g:] + host[:g]
+            acc = rot[0].copy()
+            for x in rot[1:]:
+                O.lib().orc_reduce_inplace(O.F32, acc.ctypes.data, x.ctypes.data, acc.size)
+            want = acc
+        else:
+            rc, want = O.closed_form_tree(host)
+            assert rc == 0
+        assert np.array_equal(O.bits(recv0[s:e].cpu().numpy()), O.bits(want)), "chunk %d" % c
+
+
+def test_config_2_ring_8_ranks_256mib_full_oracle():
+    world_size, n, chunk = 8, 67108864, 8388608
+    with H.World(world_size) as w:
+        send = device_inputs(world_size, n, 200, "normal")
+        recv = [G.poisoned_like(t) for t in send]
+        assert G.run_world(w, H.RING, send, recv, chunk) == 0, H.last_error()
+        # every element of every rank against the oracle's closed form on the host
+        host = [t.cpu().numpy() for t in send]
+        rc, want = O.closed_form_ring(host, chunk)
+        assert rc == 0
+        wbits = O.bits(want)
+        for r in range(world_size):
+            assert np.array_equal(O.bits(recv[r].cpu().numpy()), wbits), "rank %d" % r
+        st = w.stats(0)
+        assert st["reduce_elements"] == 58720256 and st["gather_bytes"] == 58720256 * 4
+
+
+def test_config_3_rabenseifner_16_ranks_resnet50():
+    world_size, n, chunk = 16, 102760448, 4194304
+    with H.World(world_size) as w:
+        send = device_inputs(world_size, n, 300, "normal1e-2")
+        recv = [G.poisoned_like(t) for t in send]
+        assert G.run_world(w, H.RABENSEIFNER, send, recv, chunk) == 0, H.last_error()
+        want = G.device_tree(send, (0, n))
+        for r in range(world_size):
+            assert G.bits_equal(recv[r], want), "rank %d" % r
+        check_stripes_against_oracle(send, recv[0], H.RABENSEIFNER, chunk, [0, 6, 7, 13, 14, 50, 97])
+        st = w.stats(0)
+        assert st["reduce_elements"] == 90 * 1048576  # rank 0 reduces 90 chunks
+
+
+def test_config_4_ring_small_chunks_64_streams():
+    world_size, n, chunk = 8, 16777216, 65536
+    with G.env(IBCOMM_NUM_CUDA_STREAM=64):
+        with H.World(world_size) as w:
+            send = device_inputs(world_size, n, 400, "uniform")
+            for fuse in (48, 1):
+                w.set_max_fuse(fuse)
+                recv = [G.poisoned_like(t) for t in send]
+                assert G.run_world(w, H.RING, send, recv, chunk) == 0, H.last_error()
+                check_ring_on_device(send, recv, chunk)
+            host = [t.cpu().numpy() for t in send]
+            rc, want = O.closed_form_ring(host, chunk)
+            assert np.array_equal(O.bits(recv[3].cpu().numpy()), O.bits(want))
+            assert w.stats(0)["streams_created"] == 64
+
+
+def test_config_5_ring_32_ranks_2gib_ragged_tail():
+    world_size, n, chunk = 32, 536870911, 16777216
+    free, _ = torch.cuda.mem_get_info()
+    if free < 150 * 2**30:
+        pytest.skip("needs ~140 GiB of free HBM")
+    with H.World(world_size) as w:
+        send = device_inputs(world_size, n, 500, "normal")
+        recv = [torch.empty_like(t) for t in send]
+        assert G.run_world(w, H.RING, send, recv, chunk) == 0, H.last_error()
+        check_ring_on_device(send, recv, chunk)
+        check_stripes_against_oracle(send, recv[0], H.RING, chunk, [0, 3, 4, 63, 124, 127])
+        check_stripes_against_oracle(send, recv[31], H.RING, chunk, [127])
+        del send, recv
+    torch.cuda.empty_cache()
+
+
+def test_config_1_values_cpu_shape_on_gpu():
+    # the CPU configuration's data (integers in [-1000, 1000] as float): any order gives the exact sum
+    world_size, n = 4, 4194304
+    with H.World(world_size) as w:
+        send = device_inputs(world_size, n, 100, "ints")
+        recv = [G.poisoned_like(t) for t in send]
+        assert G.run_world(w, H.RING, send, recv) == 0
+        exact = sum(t.double() for t in send).float()
+        for r in range(world_size):
+            assert torch.equal(recv[r], exact)

@@ -1,0 +1,144 @@
+"""GPU parity of the reduction kernel (stands for _reduce_inplace_cuda, allreduce_cuda_impl.h:26-33)
+through the C ABI, bit-exact against the oracle's scalar loop."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import hip_lib as H
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def oracle_add(a, b):
+    r = a.copy()
+    O.lib().orc_reduce_inplace(O.DTYPE_OF[a.dtype], r.ctypes.data, b.ctypes.data, r.size)
+    return r
+
+
+def gpu_add(a, b, off_a=0, off_b=0, off_d=0, inplace=False):
+    """a, b: host arrays; operands are placed off_* elements into 256-byte aligned device buffers."""
+    dt = O.DTYPE_OF[a.dtype]
+    n = a.size
+    ta = torch.zeros(n + 64, dtype=torch.from_numpy(a[:0]).dtype, device="cuda")
+    tb = torch.zeros_like(ta)
+    td = torch.zeros_like(ta)
+    td.view(torch.uint8).fill_(0xAB)
+    ta[off_a:off_a + n] = torch.from_numpy(a).cuda()
+    tb[off_b:off_b + n] = torch.from_numpy(b).cuda()
+    es = a.itemsize
+    dst = ta.data_ptr() + off_a * es if inplace else td.data_ptr() + off_d * es
+    torch.cuda.synchronize()
+    rc = H.lib().ibcomm_hip_reduce(dt, dst, ta.data_ptr() + off_a * es, tb.data_ptr() + off_b * es, n, None)
+    assert rc == 0, H.last_error()
+    torch.cuda.synchronize()
+    if inplace:
+        return ta[off_a:off_a + n].cpu().numpy(), None
+    full = td.cpu().numpy()
+    return full[off_d:off_d + n], full
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 3, 4, 5, 63, 64, 65, 255, 256, 257, 1023, 1025, 4099, 16384, 262144 + 3, 2097152])
+def test_f32_sizes(n):
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n).astype(np.float32)
+    b = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    got, full = gpu_add(a, b)
+    assert np.array_equal(O.bits(got), O.bits(oracle_add(a, b)))
+    assert (full.view(np.uint32)[n:] == 0xABABABAB).all(), "wrote past the end"
+
+
+@pytest.mark.parametrize("off_a,off_b,off_d", [(0, 0, 0), (1, 1, 1), (2, 2, 2), (3, 3, 3), (1, 0, 0), (0, 3, 0), (0, 0, 2), (1, 2, 3)])
+def test_f32_every_alignment_phase(off_a, off_b, off_d):
+    # chunk offsets are arbitrary element multiples, so operands can sit at any 4-byte phase
+    for n in (1, 2, 3, 4, 5, 7, 8, 9, 4097, 100003):
+        rng = np.random.default_rng(n + off_a)
+        a = rng.standard_normal(n).astype(np.float32)
+        b = rng.standard_normal(n).astype(np.float32)
+        got, full = gpu_add(a, b, off_a, off_b, off_d)
+        assert np.array_equal(O.bits(got), O.bits(oracle_add(a, b)))
+        u = full.view(np.uint32)
+        assert (u[:off_d] == 0xABABABAB).all() and (u[off_d + n:] == 0xABABABAB).all()
+
+
+def test_f32_special_values_denormals_kept():
+    tiny, dn, mx = np.float32(1e-45), np.float32(5.9e-39), np.finfo(np.float32).max
+    a = np.array([0.0, -0.0, -0.0, tiny, dn, mx, -mx, np.inf, 1.0, 16777216.0, 1e-38, 3e-39] * 50, dtype=np.float32)
+    b = np.array([-0.0, -0.0, 0.0, tiny, dn, mx, -mx, 1.0, -1.0, 1.0, -1.1e-38, 4e-39] * 50, dtype=np.float32)
+    got, _ = gpu_add(a, b)
+    want = oracle_add(a, b)
+    assert np.array_equal(O.bits(got), O.bits(want))
+    assert got[3] != 0 and got[4] != 0 and got[11] != 0  # denormal results are not flushed to zero
+
+
+def test_f32_nan_and_inf_propagate():
+    a = np.array([np.nan, 1.0, np.inf, -np.inf] * 8, dtype=np.float32)
+    b = np.array([1.0, np.nan, -np.inf, -np.inf] * 8, dtype=np.float32)
+    got, _ = gpu_add(a, b)
+    assert np.isnan(got[0::4]).all() and np.isnan(got[1::4]).all() and np.isnan(got[2::4]).all()
+    assert np.isneginf(got[3::4]).all()
+
+
+def test_in_place_is_the_reference_form():
+    # result[i] += value[i]: dst aliases the first operand
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal(70001).astype(np.float32)
+    b = rng.standard_normal(70001).astype(np.float32)
+    got, _ = gpu_add(a, b, 1, 1, 0, inplace=True)
+    assert np.array_equal(O.bits(got), O.bits(oracle_add(a, b)))
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float64, np.int64])
+def test_other_element_types(dtype):
+    rng = np.random.default_rng(3)
+    for n in (1, 2, 3, 1000, 65537):
+        if np.issubdtype(dtype, np.integer):
+            info = np.iinfo(dtype)
+            a = rng.integers(info.min, info.max, n, dtype=dtype)  # wraps on overflow like the reference's int +=
+            b = rng.integers(info.min, info.max, n, dtype=dtype)
+        else:
+            a = rng.standard_normal(n).astype(dtype)
+            b = rng.standard_normal(n).astype(dtype) * 1e-9
+        for off in (0, 1):
+            got, _ = gpu_add(a, b, off, off, off)
+            assert np.array_equal(O.bits(got), O.bits(oracle_add(a, b)))
+
+
+def test_segment_launch_matches_per_segment_results():
+    rng = np.random.default_rng(11)
+    k = H.lib().ibcomm_hip_max_segments()
+    assert k >= 32
+    sizes = [int(s) for s in rng.integers(0, 5000, k)]
+    a = [rng.standard_normal(s).astype(np.float32) for s in sizes]
+    b = [rng.standard_normal(s).astype(np.float32) for s in sizes]
+    ta = [torch.from_numpy(x).cuda() for x in a]
+    tb = [torch.from_numpy(x).cuda() for x in b]
+    td = [torch.zeros(s, dtype=torch.float32, device="cuda") for s in sizes]
+    vp = C.c_void_p
+    torch.cuda.synchronize()
+    rc = H.lib().ibcomm_hip_reduce_segments(H.F32, k, (vp * k)(*[t.data_ptr() for t in td]),
+                                            (vp * k)(*[t.data_ptr() for t in ta]), (vp * k)(*[t.data_ptr() for t in tb]),
+                                            (C.c_size_t * k)(*sizes), None)
+    assert rc == 0, H.last_error()
+    torch.cuda.synchronize()
+    for i in range(k):
+        assert np.array_equal(O.bits(td[i].cpu().numpy()), O.bits(oracle_add(a[i], b[i])))
+    assert H.lib().ibcomm_hip_reduce_segments(H.F32, k + 1, None, None, None, None, None) == H.INVALID_ARGUMENT
+
+
+def test_large_linear_property():
+    # 256 MiB operands: compare with torch's own fp32 add on the device (IEEE add, same rounding)
+    n = 67108864
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randn(n, device="cuda", generator=g)
+    b = torch.randn(n, device="cuda", generator=g)
+    d = torch.empty_like(a)
+    torch.cuda.synchronize()
+    assert H.lib().ibcomm_hip_reduce(H.F32, d.data_ptr(), a.data_ptr(), b.data_ptr(), n, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(d.view(torch.int32), (a + b).view(torch.int32))
+    # and a sampled stripe against the oracle on the host
+    s = slice(n - 100003, n)
+    assert np.array_equal(O.bits(d[s].cpu().numpy()), O.bits(oracle_add(a[s].cpu().numpy(), b[s].cpu().numpy())))
