@@ -3,6 +3,7 @@
 #include "ibcomm_hip.h"
 
 #include <new>
+#include <string>
 #include <vector>
 
 #include "backend_hip.hpp"
@@ -16,10 +17,55 @@ static_assert(IBCOMM_HIP_F32 == kF32 && IBCOMM_HIP_I32 == kI32 && IBCOMM_HIP_F64
               "dtype codes");
 static_assert(IBCOMM_HIP_RING == kRing && IBCOMM_HIP_RABENSEIFNER == kRabenseifner, "algorithm codes");
 
+// A whole-world allreduce recorded as a HIP graph.  The single-threaded driver issues the same
+// sequence of copies, launches and event edges every time it is called with the same buffers,
+// length, chunk size and knobs, so the sequence is captured once and replayed: the host then costs
+// one hipGraphLaunch instead of hundreds of launches and event calls per collective.
+struct GraphKey {
+  int algo = 0, dtype = 0, landing = 0, fuse = 0, world = 0;
+  size_t len = 0;
+  std::string chunk_env;
+  std::vector<const void*> send;
+  std::vector<void*> recv;
+  bool operator==(const GraphKey& o) const {
+    return algo == o.algo && dtype == o.dtype && landing == o.landing && fuse == o.fuse && world == o.world && len == o.len &&
+           chunk_env == o.chunk_env && send == o.send && recv == o.recv;
+  }
+};
+
+struct CachedGraph {
+  GraphKey key;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
 struct ibcomm_hip_fabric {
-  explicit ibcomm_hip_fabric(int n) : fabric(n) {}
+  explicit ibcomm_hip_fabric(int n) : fabric(n) {
+    const char* v = getenv("IBCOMM_HIP_GRAPH");
+    graph_mode = v ? atoi(v) : 1;
+    v = getenv("IBCOMM_HIP_GRAPH_MAX_OPS");
+    graph_max_ops = v ? strtoull(v, nullptr, 10) : 4096;
+  }
+  ~ibcomm_hip_fabric() {
+    DropGraphs();
+    if (origin) (void)hipStreamDestroy(origin);
+  }
+  void DropGraphs() {
+    for (CachedGraph& g : graphs) {
+      if (g.exec) (void)hipGraphExecDestroy(g.exec);
+      if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    graphs.clear();
+  }
   Fabric<HipBackend> fabric;
   int live_comms = 0;
+  int graph_mode = 1;            // 0 = always issue eagerly, 1 = capture a call shape on its second use
+  hipStream_t origin = nullptr;  // stream the graphs are captured from and replayed on
+  uint64_t graph_max_ops = 4096; // call shapes with more copies + launches than this stay eager
+  std::vector<CachedGraph> graphs;
+  GraphKey last_eager;           // shape of the most recent eagerly issued call
+  bool has_last_eager = false;
+  uint64_t graph_captures = 0, graph_replays = 0, eager_calls = 0;
 };
 
 struct ibcomm_hip_comm {
@@ -67,6 +113,8 @@ int ibcomm_hip_comm_create(ibcomm_hip_fabric* fabric, int world_size, ibcomm_hip
 int ibcomm_hip_comm_destroy(ibcomm_hip_comm* comm) {
   if (!comm) return kOk;
   comm->comm.Abort();
+  comm->owner->DropGraphs();  // recorded graphs point into this communicator's pool
+  comm->owner->has_last_eager = false;
   comm->owner->live_comms--;
   delete comm;
   return kOk;
@@ -103,6 +151,60 @@ int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* c, const int32_t* s, 
   return ibcomm_hip_allreduce_rabenseifner(c, kI32, s, r, n);
 }
 
+namespace {
+
+constexpr size_t kMaxCachedGraphs = 16;
+
+uint64_t DeviceOps(const EngineStats& s) { return s.reduce_launches + s.landing_copies + s.gather_copies; }
+
+int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g) {
+  IBCOMM_HIP_CHECK(hipGraphLaunch(g.exec, f->origin));
+  IBCOMM_HIP_CHECK(hipStreamSynchronize(f->origin));
+  f->graph_replays++;
+  return kOk;
+}
+
+// Records one RunWorld() into a graph.  While recording, every rank issues all of its work on the
+// one capturing stream, so the graph is a single ordered chain of kernels in the (dependency
+// respecting) order the driver issues them.  A chain is what the runtime handles well: recording
+// the ranks' own multi-stream, event-linked work gave graphs whose instantiation did not finish.
+// Launches at the default fusion are large enough to fill the GPU on their own, so the chain costs
+// little overlap and removes the host's launch and event work from every later call.
+int CaptureWorld(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key,
+                 const void* const* sendbufs, void* const* recvbufs, CachedGraph* out) {
+  if (!f->origin) IBCOMM_HIP_CHECK(hipStreamCreateWithFlags(&f->origin, hipStreamNonBlocking));
+  for (auto* c : cs) c->pool().OverrideStream(f->origin);
+  hipError_t e = hipStreamBeginCapture(f->origin, hipStreamCaptureModeRelaxed);
+  int rc = kOk;
+  if (e != hipSuccess) {
+    rc = Fail(kDeviceError, "hipStreamBeginCapture failed: %s", hipGetErrorString(e));
+  } else {
+    rc = RunWorld<HipBackend>(cs.data(), key.world, key.algo, key.dtype, sendbufs, recvbufs, key.len, false);
+  }
+  for (auto* c : cs) c->pool().ClearOverride();
+  if (e != hipSuccess) return rc;
+  hipGraph_t graph = nullptr;
+  e = hipStreamEndCapture(f->origin, &graph);
+  if (rc != kOk) {
+    if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+  }
+  if (e != hipSuccess || !graph) return Fail(kDeviceError, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return Fail(kDeviceError, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  out->key = key;
+  out->graph = graph;
+  out->exec = exec;
+  f->graph_captures++;
+  return kOk;
+}
+
+}  // namespace
+
 int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
                                const void* const* sendbufs, void* const* recvbufs, size_t len) {
   if (!comms || !sendbufs || !recvbufs || world_size < 1) return Fail(kInvalidArgument, "null argument");
@@ -112,7 +214,76 @@ int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, in
     if (comms[r]->owner != comms[0]->owner) return Fail(kInvalidArgument, "communicators belong to different fabrics");
     cs[r] = &comms[r]->comm;
   }
-  return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+  ibcomm_hip_fabric* f = comms[0]->owner;
+  // Recording hipMemcpyAsync device-to-device copies into a graph crashed the host process inside
+  // the runtime on ROCm 7.2 (gfx950), so the per-message-memcpy landing mode is never recorded.
+  if (f->graph_mode == 0 || world_size == 1 || cs[0]->landing() == kLandMemcpy) {
+    f->eager_calls++;
+    return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+  }
+
+  GraphKey key;
+  key.algo = algo;
+  key.dtype = dtype;
+  key.landing = cs[0]->landing();
+  key.fuse = cs[0]->max_fuse();
+  key.world = world_size;
+  key.len = len;
+  const char* env = getenv("IBCOMM_CHUNKSIZE");  // read on every call, like the reference
+  key.chunk_env = env ? env : "";
+  key.send.assign(sendbufs, sendbufs + world_size);
+  key.recv.assign(recvbufs, recvbufs + world_size);
+  for (int r = 1; r < world_size; r++)
+    if (cs[r]->landing() != key.landing || cs[r]->max_fuse() != key.fuse) key.fuse = -1 - r;  // mixed knobs: never equal
+
+  for (CachedGraph& g : f->graphs)
+    if (g.key == key) return ReplayGraph(f, g);
+
+  if (f->has_last_eager && f->last_eager == key) {
+    // Second call with this shape: record it.  The recording itself executes nothing, so launch it once.
+    CachedGraph g;
+    const int rc = CaptureWorld(f, cs, key, sendbufs, recvbufs, &g);
+    if (rc != kOk) {
+      for (auto* c : cs) c->Abort();
+      f->fabric.Reset();
+      f->fabric.EndLockstep();
+      f->has_last_eager = false;
+      return rc;
+    }
+    if (f->graphs.size() >= kMaxCachedGraphs) {
+      (void)hipGraphExecDestroy(f->graphs.front().exec);
+      (void)hipGraphDestroy(f->graphs.front().graph);
+      f->graphs.erase(f->graphs.begin());
+    }
+    f->graphs.push_back(g);
+    return ReplayGraph(f, f->graphs.back());
+  }
+
+  f->eager_calls++;
+  uint64_t ops_before = 0, ops_after = 0;
+  for (auto* c : cs) ops_before += DeviceOps(c->stats());
+  const int rc = RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+  for (auto* c : cs) ops_after += DeviceOps(c->stats());
+  // Only shapes of a bounded number of device operations are recorded on their next use.
+  f->has_last_eager = (rc == kOk) && (ops_after - ops_before <= f->graph_max_ops);
+  if (rc == kOk) f->last_eager = key;
+  return rc;
+}
+
+int ibcomm_hip_fabric_graph_counters(ibcomm_hip_fabric* fabric, uint64_t* eager_calls, uint64_t* captures, uint64_t* replays) {
+  if (!fabric) return Fail(kInvalidArgument, "fabric is null");
+  if (eager_calls) *eager_calls = fabric->eager_calls;
+  if (captures) *captures = fabric->graph_captures;
+  if (replays) *replays = fabric->graph_replays;
+  return kOk;
+}
+
+int ibcomm_hip_fabric_set_graph_mode(ibcomm_hip_fabric* fabric, int mode) {
+  if (!fabric) return Fail(kInvalidArgument, "fabric is null");
+  if (mode != 0 && mode != 1) return Fail(kInvalidArgument, "graph mode must be 0 or 1");
+  fabric->graph_mode = mode;
+  if (mode == 0) fabric->DropGraphs();
+  return kOk;
 }
 
 int ibcomm_hip_reduce(int dtype, void* dst, const void* a, const void* b, size_t n, void* stream) {

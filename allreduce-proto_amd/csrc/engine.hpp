@@ -10,8 +10,9 @@
 //     this rank consumes and emits;
 //   * Progress() walks the plan without ever waiting for the device: it posts
 //     every send whose data has been *enqueued*, takes every message a peer
-//     has posted, lands it in a pool slot (hipMemcpyAsync by default), and
-//     launches one segment kernel over all chunks that landed in this pass:
+//     has posted, lands it in a pool slot (one copy-kernel launch for all of
+//     them by default, or one hipMemcpyAsync each), and launches one segment
+//     kernel over all chunks that landed in this pass:
 //         recvbuf[c] = incoming + sendbuf[c]     ring steps, first halving step
 //         recvbuf[c] = incoming + recvbuf[c]     later halving steps
 //     Finished chunks of the gather phase land straight in recvbuf and are
@@ -99,8 +100,8 @@ class Communicator {
     if (max_fuse_ < 1 || max_fuse_ > kMaxSegments)
       return Fail(kInvalidArgument, "IBCOMM_HIP_MAX_FUSE must be in [1, %d]", kMaxSegments);
     v = getenv("IBCOMM_HIP_LANDING");
-    if (!v || !strcmp(v, "memcpy")) landing_ = kLandMemcpy;
-    else if (!strcmp(v, "kernel")) landing_ = kLandKernel;
+    if (!v || !strcmp(v, "kernel")) landing_ = kLandKernel;
+    else if (!strcmp(v, "memcpy")) landing_ = kLandMemcpy;
     else if (!strcmp(v, "direct")) landing_ = kLandDirect;
     else return Fail(kInvalidArgument, "IBCOMM_HIP_LANDING must be memcpy, kernel or direct, not '%s'", v);
     // The working GPU buffer (IBCOMM_WORK_GPU_MEMORY_SIZE, ibverbs_communicator_cuda.cpp:12-33) held
@@ -327,7 +328,7 @@ class Communicator {
     return B::StreamWaitEvent(s, st.event);
   }
   int WaitOnMessage(Stream s, const Message& m) {
-    if (!m.has_ready) return kOk;
+    if (!m.has_ready || m.ready_stream == s) return kOk;
     stats_.stream_waits++;
     return B::StreamWaitEvent(s, m.ready);
   }
@@ -350,7 +351,7 @@ class Communicator {
           p.issued = true;
           p.has_event = c.has_done;
           p.event = c.done;
-          p.stream = Stream{};
+          p.stream = c.done_stream;
         }
         *moved = true;
       }
@@ -363,6 +364,7 @@ class Communicator {
       const SendOp& s = plan_.sends[next_send_];
       const void* src;
       Event ready{};
+      Stream ready_stream{};
       bool has_ready = false;
       if (s.dep < 0) {
         src = SendPtr(s.chunk);
@@ -371,9 +373,10 @@ class Communicator {
         if (!d.issued) break;  // the data has not been enqueued yet
         src = RecvPtr(s.chunk);
         ready = d.event;
+        ready_stream = d.stream;
         has_ready = d.has_event;
       }
-      const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready);
+      const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready, ready_stream);
       posted_[s.peer].push_back(PostedSend{ticket, static_cast<int>(next_send_)});
       if (s.dep >= 0 || in_place_) chunk_unconsumed_[s.chunk]++;
       outstanding_sends_++;
@@ -421,7 +424,7 @@ class Communicator {
   // Finished chunks: recvbuf[c] <- message.
   int FlushGathers() {
     if (pending_gather_.empty()) return kOk;
-    if (landing_ == kLandKernel) {
+    if (landing_ != kLandMemcpy) {
       Stream s;
       IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
       SegmentBatch batch;
@@ -440,7 +443,7 @@ class Communicator {
       IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
       for (const PendingRecv& p : pending_gather_) {
         const RecvOp& r = plan_.recvs[p.op];
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
         recv_done_[p.op] = done;
         chunk_last_[r.chunk] = done;
       }
@@ -458,7 +461,7 @@ class Communicator {
         stats_.gather_bytes += ChunkBytes(c);
         OpState done;
         IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
         recv_done_[p.op] = done;
         chunk_last_[c] = done;
       }
@@ -486,7 +489,7 @@ class Communicator {
         stats_.landing_copies++;
         stats_.landing_bytes += ChunkBytes(r.chunk);
         IBCOMM_RETURN_IF_ERROR(RecordEvent(si, &landed[i]));
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, landed[i].event, true);
+        fabric_->Complete(rank_, r.peer, p.msg.ticket, landed[i].event, true, landed[i].stream);
       }
       s = landed[0].stream;
       for (size_t i = 1; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOn(s, landed[i]));
@@ -509,7 +512,7 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
         for (size_t i = 0; i < n; i++) {
           const PendingRecv& p = pending_reduce_[i];
-          fabric_->Complete(rank_, plan_.recvs[p.op].peer, p.msg.ticket, done.event, true);
+          fabric_->Complete(rank_, plan_.recvs[p.op].peer, p.msg.ticket, done.event, true, done.stream);
         }
       }
     }
@@ -542,7 +545,7 @@ class Communicator {
       recv_done_[p.op] = done;
       chunk_last_[r.chunk] = done;
       if (p.slot) controller_.returnMemory(p.slot, done.event, s);
-      if (landing_ == kLandDirect) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true);
+      if (landing_ == kLandDirect) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
       chunk_in_batch_[r.chunk] = 0;
     }
     pending_reduce_.clear();
@@ -561,7 +564,7 @@ class Communicator {
   MemoryPool<B> pool_;
   MemoryController<B> controller_;
   int max_fuse_ = kMaxSegments;
-  int landing_ = kLandMemcpy;
+  int landing_ = kLandKernel;
   long long work_gpu_memory_size_ = 0;
 
   bool active_ = false;

@@ -40,12 +40,14 @@ class Fabric {
     size_t bytes = 0;
     typename B::Event ready{};
     bool has_ready = false;
+    typename B::Stream ready_stream{};  // stream `ready` was recorded on (a wait from that same stream is redundant)
     uint64_t ticket = 0;
   };
   struct Completion {
     uint64_t ticket = 0;
     typename B::Event done{};
     bool has_done = false;
+    typename B::Stream done_stream{};
   };
 
   explicit Fabric(int world_size) : n_(world_size), channels_(static_cast<size_t>(world_size) * world_size) {
@@ -54,7 +56,8 @@ class Fabric {
 
   int world_size() const { return n_; }
 
-  uint64_t PostSend(int from, int to, const void* src, size_t bytes, typename B::Event ready, bool has_ready) {
+  uint64_t PostSend(int from, int to, const void* src, size_t bytes, typename B::Event ready, bool has_ready,
+                    typename B::Stream ready_stream = typename B::Stream{}) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
     Message m;
@@ -62,6 +65,7 @@ class Fabric {
     m.bytes = bytes;
     m.ready = ready;
     m.has_ready = has_ready;
+    m.ready_stream = ready_stream;
     m.ticket = c.next_ticket++;
     c.inbox.push_back(m);
     c.posted++;
@@ -73,21 +77,41 @@ class Fabric {
   bool Take(int to, int from, Message* out) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
-    if (c.inbox.empty()) return false;
+    if (c.inbox.empty() || c.inbox.front().ticket >= c.visible_below) return false;
     *out = c.inbox.front();
     c.inbox.pop_front();
     c.taken++;
     return true;
   }
 
+  // Lockstep emulation for a single-threaded driver.  Real ranks run at the same time, so what a
+  // rank can receive at some instant does not depend on the order a driver happens to visit the
+  // ranks in.  BeginSweep() freezes, for every channel, the set of receivable messages to those
+  // posted so far; messages posted during the sweep become receivable at the next BeginSweep().
+  // EndLockstep() lifts the limit (the threaded, one-thread-per-rank use never sets it).
+  void BeginSweep() {
+    for (auto& c : channels_) {
+      std::lock_guard<std::mutex> lock(c->mu);
+      c->visible_below = c->next_ticket;
+    }
+  }
+  void EndLockstep() {
+    for (auto& c : channels_) {
+      std::lock_guard<std::mutex> lock(c->mu);
+      c->visible_below = UINT64_MAX;
+    }
+  }
+
   // Receiver: the pull of message `ticket` has been enqueued; `done` completes when it has read the source.
-  void Complete(int to, int from, uint64_t ticket, typename B::Event done, bool has_done) {
+  void Complete(int to, int from, uint64_t ticket, typename B::Event done, bool has_done,
+                typename B::Stream done_stream = typename B::Stream{}) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
     Completion k;
     k.ticket = ticket;
     k.done = done;
     k.has_done = has_done;
+    k.done_stream = done_stream;
     c.completions.push_back(k);
     c.delivered++;
   }
@@ -134,6 +158,7 @@ class Fabric {
     std::deque<Message> inbox;
     std::deque<Completion> completions;
     uint64_t next_ticket = 0;
+    uint64_t visible_below = UINT64_MAX;
     uint64_t posted = 0;
     uint64_t taken = 0;
     uint64_t delivered = 0;

@@ -133,8 +133,20 @@ class MemoryPool {
     return kOk;
   }
 
+  // While set, NextStream() hands out this one stream only.  Used to record a collective as a
+  // single ordered chain of device work (a HIP graph without cross-stream edges).
+  void OverrideStream(typename B::Stream s) {
+    override_ = s;
+    has_override_ = true;
+  }
+  void ClearOverride() { has_override_ = false; }
+
   // Round-robin over at most max_streams() streams, created on first use.
   int NextStream(typename B::Stream* out) {
+    if (has_override_) {
+      *out = override_;
+      return kOk;
+    }
     if (static_cast<int>(streams_.size()) < max_streams_ && cursor_ >= streams_.size()) {
       typename B::Stream s;
       IBCOMM_RETURN_IF_ERROR(B::StreamCreate(&s));
@@ -205,6 +217,8 @@ class MemoryPool {
   std::vector<typename B::Stream> streams_;
   size_t cursor_ = 0;
   bool controller_in_use_ = false;
+  typename B::Stream override_{};
+  bool has_override_ = false;
 };
 
 template <class B>

@@ -6,7 +6,7 @@
 
 namespace ibcomm_hip {
 
-constexpr int kMaxSegments = 48;  // 48 * 40 B of kernel arguments, well under the 4 KiB limit
+constexpr int kMaxSegments = 64;  // 64 * 40 B of kernel arguments, under the 4 KiB limit
 
 struct Segment {
   void* dst;        // written

@@ -4,6 +4,12 @@
 // ranks on one GPU a single thread can do the same job deterministically: call Progress() on each
 // rank in turn until all have issued their whole plan.  Progress() never waits, so a full sweep in
 // which no rank moved means the plans do not fit together; that is reported instead of spinning.
+//
+// Sweeps are lockstep: during a sweep a rank can take only the messages that had been posted when
+// the sweep began (Fabric::BeginSweep).  Without that, the rank visited last would find its
+// upstream's entire reduce-scatter already posted and the emulated ranks would run one after the
+// other; with it every sweep is one step of the algorithm on all ranks at once, and their launches
+// are independent and overlap on the GPU the way N devices would work side by side.
 #pragma once
 
 #include <vector>
@@ -33,8 +39,10 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
   if (rc == kOk) {
     std::vector<char> done(n, 0);
     int remaining = n;
+    Fabric<B>* fabric = comms[0]->fabric();
     while (remaining > 0 && rc == kOk) {
       bool any = false;
+      fabric->BeginSweep();
       for (int r = 0; r < n && rc == kOk; r++) {
         if (done[r]) continue;
         bool progressed = false, finished = false;
@@ -45,6 +53,7 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
           remaining--;
         }
       }
+      // a sweep sees everything posted before it began, so one idle sweep is conclusive
       if (rc == kOk && remaining > 0 && !any) {
         int stuck = 0;
         while (done[stuck]) stuck++;
@@ -54,6 +63,7 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
       }
     }
   }
+  comms[0]->fabric()->EndLockstep();
   if (rc != kOk) {
     // keep the message of the first failure
     char saved[512];

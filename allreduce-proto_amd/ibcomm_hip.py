@@ -26,7 +26,7 @@ EXPORTS = [
     "ibcomm_hip_reduce", "ibcomm_hip_reduce_segments", "ibcomm_hip_max_segments", "ibcomm_hip_split_buffer",
     "ibcomm_hip_rank_to_chunk", "ibcomm_hip_get_exp_of_two", "ibcomm_hip_plan_create", "ibcomm_hip_plan_destroy",
     "ibcomm_hip_plan_counts", "ibcomm_hip_plan_range", "ibcomm_hip_plan_recv", "ibcomm_hip_plan_send",
-    "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
+    "ibcomm_hip_fabric_set_graph_mode", "ibcomm_hip_fabric_graph_counters", "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
 ]
 
 
@@ -74,6 +74,8 @@ def lib():
     L.ibcomm_hip_plan_range.argtypes = [vp, i, C.POINTER(sz), C.POINTER(sz)]
     L.ibcomm_hip_plan_recv.argtypes = [vp, i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_plan_send.argtypes = [vp, i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
+    L.ibcomm_hip_fabric_set_graph_mode.argtypes = [vp, i]
+    L.ibcomm_hip_fabric_graph_counters.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
     L.ibcomm_hip_comm_set_max_fuse.argtypes = [vp, i]
     L.ibcomm_hip_comm_set_landing.argtypes = [vp, i]
     L.ibcomm_hip_comm_stats.argtypes = [vp, C.POINTER(Stats)]
@@ -152,6 +154,15 @@ class World:
                 raise RuntimeError("comm_create: %d %s" % (rc, last_error()))
             L.ibcomm_hip_comm_register_myself(h, r)
             self.comms.append(h)
+
+    def set_graph_mode(self, mode):
+        assert lib().ibcomm_hip_fabric_set_graph_mode(self.fabric, mode) == 0, last_error()
+
+    def graph_counters(self):
+        """-> (eager calls, graphs captured, graph replays) of the single-thread driver."""
+        a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert lib().ibcomm_hip_fabric_graph_counters(self.fabric, C.byref(a), C.byref(b), C.byref(c)) == 0
+        return a.value, b.value, c.value
 
     def set_max_fuse(self, f):
         for h in self.comms:

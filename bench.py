@@ -181,6 +181,7 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
     ap.add_argument("--landing", choices=["memcpy", "kernel", "direct"], default=None)
     ap.add_argument("--fuse", type=int, default=None)
+    ap.add_argument("--no-graph", action="store_true", help="issue every step eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
     args = ap.parse_args()
@@ -214,22 +215,28 @@ def main():
             w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT}[args.landing])
         if args.fuse:
             w.set_max_fuse(args.fuse)
-        for _ in range(args.warmup):
+        if args.no_graph:
+            w.set_graph_mode(0)
+        # one eagerly issued step to read the per-step work counters (graph replays bypass them)
+        w.reset_stats()
+        assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0, H.last_error()
+        st = [w.stats(r) for r in range(world)]
+        # untimed: at least two more calls so that the call shape is recorded before timing starts
+        for _ in range(max(args.warmup, 0 if args.no_graph else 2)):
             assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0, H.last_error()
         torch.cuda.synchronize()
-        w.reset_stats()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             rc = w.allreduce_ptrs(algo, H.F32, sp, rp, n)
             assert rc == 0, H.last_error()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        st = [w.stats(r) for r in range(world)]
+        graph_counters = w.graph_counters()
 
     sec_per_step = (t1 - t0) / args.steps
     parity = check_result(torch, O, H, algo, send, recv, chunk)
 
-    steps = args.steps
+    steps = 1  # the counters in `st` cover exactly one step
     total = {k: sum(s[k] for s in st) for k in st[0]}
     device_bytes_per_step = (12 * total["reduce_elements"] + 2 * total["landing_bytes"] + 2 * total["gather_bytes"]) / steps
     segs_per_launch = max(1, round(st[0]["reduce_segments"] / max(1, st[0]["reduce_launches"])))
@@ -254,8 +261,8 @@ def main():
                         "IBCOMM_CHUNKSIZE=%d, all ranks' schedules executed per step" % (
                             args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk),
             "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk,
-            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "memcpy"),
-            "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "48")),
+            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "kernel"),
+            "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64")),
         },
         "parity_bit_exact": parity,
         "extra": {
@@ -270,6 +277,8 @@ def main():
             "rank0_landing_copies_per_step": st[0]["landing_copies"] / steps,
             "rank0_gather_copies_per_step": st[0]["gather_copies"] / steps,
             "streams_per_rank": st[0]["streams_created"],
+            "issue": "eager" if args.no_graph else "hip graph replay",
+            "graph_calls_eager_captured_replayed": list(graph_counters),
             "pool_slots_high_water": max(s["slots_high_water"] for s in st),
         },
     }

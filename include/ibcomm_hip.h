@@ -103,6 +103,14 @@ int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* comm, const int32_t* 
 int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
                                const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
 
+/* ibcomm_hip_world_allreduce records the device work of a call shape (same buffers, length, chunk
+ * size and knobs) into a HIP graph on its second use and replays the graph from then on; mode 0
+ * turns that off (every call is issued eagerly), mode 1 is the default (IBCOMM_HIP_GRAPH).  No
+ * counterpart in the reference, whose host loop re-issues every operation on every call. */
+int ibcomm_hip_fabric_set_graph_mode(ibcomm_hip_fabric* fabric, int mode);
+int ibcomm_hip_fabric_graph_counters(ibcomm_hip_fabric* fabric, uint64_t* eager_calls, uint64_t* captures,
+                                     uint64_t* replays);
+
 /* The reduction kernel on its own, asynchronous on `stream` (a hipStream_t, NULL = default
  * stream): dst[i] = a[i] + b[i].  Stands for _reduce_inplace_cuda<T>
  * (ibcomm/allreduce_cuda_impl.h:26-33, launches at :132-133 and :510-512), which is the case

@@ -142,11 +142,12 @@ def test_work_per_rank_matches_the_schedule():
     assert st.reduce_elements == (world - 1) * n // world
     assert st.gather_bytes == (world - 1) * n // world * 4
     assert st.messages_received == 2 * (world - 1) * q and st.messages_sent == 2 * (world - 1) * q
-    # fused: whatever has landed goes into one launch (how much that is depends on the order in
-    # which the driver visits the ranks), never more than 48 chunks
+    # fused: the driver steps all ranks in lockstep, so each pass sees exactly one ring step's
+    # group (64 chunks here) and reduces it with as few launches as the segment limit allows
+    rep = check(RING, bufs, chunk, max_fuse=64)
+    assert rep.rank0.reduce_launches == world - 1 and rep.rank0.reduce_segments == (world - 1) * q
     rep = check(RING, bufs, chunk, max_fuse=48)
-    assert -(-(world - 1) * q // 48) <= rep.rank0.reduce_launches <= world
-    assert rep.rank0.reduce_segments == (world - 1) * q
+    assert rep.rank0.reduce_launches == 2 * (world - 1)
     # Rabenseifner rank 0 of 4: halving windows of 2 and 1 groups
     rep = check(RABEN, bufs, chunk, max_fuse=1)
     assert rep.rank0.reduce_segments == 3 * q and rep.rank0.gather_bytes == 3 * q * chunk

@@ -89,6 +89,43 @@ def test_odd_chunk_offsets_keep_vector_path_correct():
         G.check_against_oracle(w, H.RING, rand_bufs(5, 1003))
 
 
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 4, None), (H.RING, 8, 4096), (H.RABENSEIFNER, 8, None)])
+def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
+    # the single-thread driver records a call shape on its second use and replays it afterwards;
+    # every replay must give what an eager run gives, with other device work in between
+    n = 262144 + 3
+    with H.World(world_size) as w:
+        w.set_landing(landing)
+        w.set_max_fuse(5)
+        send = [torch.empty(n, device="cuda") for _ in range(world_size)]
+        recv = [torch.empty(n, device="cuda") for _ in range(world_size)]
+        scratch = torch.zeros(1 << 20, device="cuda")
+        for it in range(7):
+            host = rand_bufs(world_size, n, seed=100 * it)
+            for t, h in zip(send, host):
+                t.copy_(torch.from_numpy(h))
+            for t in recv:
+                t.view(torch.uint8).fill_(0x55)
+            scratch.add_(1.0).mul_(0.5)  # unrelated eager work between replays
+            assert G.run_world(w, algo, send, recv, chunk) == 0, H.last_error()
+            orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
+            assert orc == 0
+            for r in range(world_size):
+                assert np.array_equal(O.bits(recv[r].cpu().numpy()), O.bits(want[r])), "call %d rank %d" % (it, r)
+        eager, captured, replayed = w.graph_counters()
+        if landing == H.LAND_MEMCPY:  # per-message hipMemcpyAsync is never recorded
+            assert (eager, captured, replayed) == (7, 0, 0)
+        else:
+            assert (eager, captured, replayed) == (1, 1, 6)
+        # a different shape is a different graph; graph mode 0 goes back to eager issue
+        G.check_against_oracle(w, algo, rand_bufs(world_size, 5000, seed=1))
+        w.set_graph_mode(0)
+        for _ in range(2):
+            assert G.run_world(w, algo, send, recv, chunk) == 0
+        assert w.graph_counters()[0] == eager + 3
+
+
 # ------------------------------------------------------------------ reference tester cases
 
 def run_kat(world_size, algo, n, chunk=None):
