@@ -25,7 +25,9 @@ __device__ __forceinline__ void StoreVec(V* p, V v) {
 // One workgroup column (blockIdx.y) per segment; blockIdx.x strides over tiles
 // of THREADS * UNROLL 16-byte vectors.  T is the element type, V the 16-byte
 // vector of T.  Integer types are instantiated unsigned so that += wraps.
-template <typename T, typename V, int THREADS, int UNROLL, bool NT>
+// ADD selects dst = a + b; otherwise the launch is a copy, dst = a.  The two are
+// separate kernels so that a profile tells reductions from landing copies.
+template <typename T, typename V, int THREADS, int UNROLL, bool NT, bool ADD>
 __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batch) {
   const Segment s = batch.seg[blockIdx.y];
   const uint64_t n = s.n;
@@ -35,7 +37,7 @@ __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batc
   T* dst2 = static_cast<T*>(s.dst2);
   const T* a = static_cast<const T*>(s.a);
   const T* b = static_cast<const T*>(s.b);
-  const bool has_b = (b != nullptr);
+  constexpr bool has_b = ADD;
   const bool has_d2 = (dst2 != nullptr);
 
   constexpr uint64_t kPerVec = 16 / sizeof(T);
@@ -111,7 +113,10 @@ namespace {
 
 template <typename T, typename V, int THREADS, int UNROLL, bool NT>
 hipError_t LaunchOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
-  hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, UNROLL, NT>), grid, dim3(THREADS), 0, stream, batch);
+  if (batch.seg[0].b != nullptr)
+    hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, UNROLL, NT, true>), grid, dim3(THREADS), 0, stream, batch);
+  else
+    hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, UNROLL, NT, false>), grid, dim3(THREADS), 0, stream, batch);
   return hipGetLastError();
 }
 
@@ -167,9 +172,11 @@ hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuni
   if (es == 0) return hipErrorInvalidValue;
 
   uint64_t max_n = 0;
+  const bool add = batch.seg[0].b != nullptr;
   for (int i = 0; i < batch.count; i++) {
     const Segment& s = batch.seg[i];
     if (s.n && (!s.dst || !s.a)) return hipErrorInvalidValue;
+    if ((s.b != nullptr) != add) return hipErrorInvalidValue;  // a launch is all adds or all copies
     if (s.n > max_n) max_n = s.n;
   }
   if (max_n == 0) return hipSuccess;

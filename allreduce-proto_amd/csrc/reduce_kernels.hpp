@@ -39,7 +39,8 @@ struct LaunchTuning {
 
 LaunchTuning DefaultTuning();
 
-// Enqueue one launch covering batch.seg[0..count).  Empty segments are legal.
+// Enqueue one launch covering batch.seg[0..count).  Empty segments are legal; all segments of a
+// launch must be of one kind (every b set: add, every b null: copy).
 // Returns the HIP error of the launch.
 hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuning& tuning, hipStream_t stream);
 

@@ -1,0 +1,134 @@
+// Drop-in for PFNProto's ibcomm/ibverbs_communicator.h on one MI355X.
+//
+// Same class name, constructor, connection-management calls and allreduce member templates as the
+// reference (ibcomm/ibverbs_communicator.h:59-123), implemented over the C ABI of libibcomm_hip.so.
+// The InfiniBand network is replaced by an in-process loopback: every communicator constructed with
+// the same world size in one process joins the same loopback world, and each emulated rank calls the
+// blocking allreduce from a thread of its own, the way each process does in the reference.
+//
+//   IBVerbsCommunicator comm(world_size);          // ibverbs_communicator.cpp:24-99
+//   comm.RegisterMyself(rank);                     // :355-357
+//   comm.AllreduceRingCuda(send_dev, recv_dev, n); // allreduce_cuda_impl.h:35-301
+//
+// Failures behave as in the reference: a message on stderr and exit(code) with the codes of
+// ibcomm/util.h:32-42.  Element types: float, double, 32- and 64-bit integers.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <map>
+#include <mutex>
+#include <type_traits>
+
+#include "ibcomm/util.h"
+#include "ibcomm_hip.h"
+
+struct ProcessInfo {  // ibverbs_communicator.h:23-27; carries nothing over the loopback
+  uint16_t lid;
+  uint32_t qp_n;
+  uint32_t psn;
+};
+
+class IBVerbsCommunicator {
+ public:
+  IBVerbsCommunicator() {}
+  explicit IBVerbsCommunicator(int world_size) { Init(world_size); }
+  IBVerbsCommunicator(const IBVerbsCommunicator&) = delete;
+  IBVerbsCommunicator& operator=(const IBVerbsCommunicator&) = delete;
+  IBVerbsCommunicator(IBVerbsCommunicator&&) = delete;
+  IBVerbsCommunicator& operator=(IBVerbsCommunicator&&) = delete;
+
+  ~IBVerbsCommunicator() {
+    if (!comm_) return;
+    ibcomm_hip_comm_destroy(comm_);
+    Registry& reg = registry();
+    std::lock_guard<std::mutex> lock(reg.mu);
+    World& w = reg.worlds[world_size_];
+    if (--w.users == 0) {
+      ibcomm_hip_fabric_destroy(w.fabric);
+      reg.worlds.erase(world_size_);
+    }
+  }
+
+  void Init(int world_size) {
+    if (comm_) {
+      util::IbcommWarning(__FILE__, __LINE__, "IBVerbsCommunicator is already initialized.");
+      return;
+    }
+    Registry& reg = registry();
+    std::lock_guard<std::mutex> lock(reg.mu);
+    World& w = reg.worlds[world_size];
+    if (!w.fabric) Check(ibcomm_hip_fabric_create(world_size, &w.fabric), __LINE__);
+    Check(ibcomm_hip_comm_create(w.fabric, world_size, &comm_), __LINE__);
+    w.users++;
+    world_size_ = world_size;
+  }
+
+  // Queue-pair bring-up (ibverbs_communicator.cpp:286-353) has nothing to exchange in one process.
+  struct ProcessInfo RegisterProcess(int, struct ProcessInfo) { return ProcessInfo{0, 0, 0}; }
+  struct ProcessInfo CreateQueuePair(int) { return ProcessInfo{0, 0, 0}; }
+  void RegisterQueuePair(int, struct ProcessInfo) {}
+  void RegisterMyself(int my_rank) {
+    my_rank_ = my_rank;
+    Check(ibcomm_hip_comm_register_myself(comm_, my_rank), __LINE__);
+  }
+
+  // Device buffers.  Blocking; every rank of the world must be inside the same call.
+  template <typename T>
+  void AllreduceRingCuda(const T* sendbuf, T* recvbuf, size_t len_elements) {
+    Check(ibcomm_hip_allreduce_ring(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
+  }
+  template <typename T>
+  void AllreduceRabenseifnerCuda(const T* sendbuf, T* recvbuf, size_t len_elements) {
+    Check(ibcomm_hip_allreduce_rabenseifner(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
+  }
+
+  // The host-buffer variants (ibcomm/allreduce_cpu_impl.h) are the reference's CPU path; this build
+  // accelerates the device path only.
+  template <typename T>
+  void AllreduceRing(const T*, T*, size_t) {
+    util::IbcommError(__FILE__, __LINE__, util::IBCOMM_ERROR_CODE::NOT_SUPPORTED,
+                      "AllreduceRing on host buffers is not part of the HIP build; use AllreduceRingCuda.");
+  }
+  template <typename T>
+  void AllreduceRabenseifner(const T*, T*, size_t) {
+    util::IbcommError(__FILE__, __LINE__, util::IBCOMM_ERROR_CODE::NOT_SUPPORTED,
+                      "AllreduceRabenseifner on host buffers is not part of the HIP build; use AllreduceRabenseifnerCuda.");
+  }
+
+  ibcomm_hip_comm* handle() { return comm_; }
+
+ private:
+  struct World {
+    ibcomm_hip_fabric* fabric = nullptr;
+    int users = 0;
+  };
+  struct Registry {
+    std::mutex mu;
+    std::map<int, World> worlds;
+  };
+  static Registry& registry() {
+    static Registry r;
+    return r;
+  }
+
+  template <typename T>
+  static constexpr int DType() {
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value ||
+                      (std::is_integral<T>::value && (sizeof(T) == 4 || sizeof(T) == 8)),
+                  "allreduce element type must be float, double or a 32/64-bit integer");
+    return std::is_same<T, float>::value ? IBCOMM_HIP_F32
+           : std::is_same<T, double>::value ? IBCOMM_HIP_F64
+           : sizeof(T) == 4 ? IBCOMM_HIP_I32
+                            : IBCOMM_HIP_I64;
+  }
+
+  static void Check(int rc, int line) {
+    if (rc == 0) return;
+    util::IbcommError(__FILE__, line, static_cast<util::IBCOMM_ERROR_CODE>(rc), "%s", ibcomm_hip_last_error());
+  }
+
+  ibcomm_hip_comm* comm_ = nullptr;
+  int my_rank_ = -1;
+  int world_size_ = 0;
+};

@@ -31,6 +31,11 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per launch of the reduction kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
+# each calibrated against a device copy of known size; the summary with the commands is
+# profiles/segment_kernel_add_ring8_256MiB.md.  Shapes that have not been measured report null.
+MEASURED_TRAFFIC_BYTES = {"4 segments x 2097152 fp32": 100693387}
+
 CONFIGS = {
     # id: (algo name, ranks, elements per rank, IBCOMM_CHUNKSIZE, data)
     2: ("ring", 8, 67108864, 8388608, "normal"),
@@ -99,7 +104,9 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
     vp = C.c_void_p
     n = send[0].numel()
     per_buf = max(1, n // seg_elems)
-    # rotate through the ranks' buffers so that successive launches touch different memory
+    # Every operand of every segment is a distinct range, and successive launches walk through
+    # all ranks' buffers (several GiB), so nothing is served from a cache: dst and a come from
+    # rank r's recvbuf / sendbuf, b from another rank's recvbuf at the same offset.
     shapes = []
     for i in range(world * 2):
         dst, a, b = [], [], []
@@ -109,7 +116,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
             off = ((idx // world) % per_buf) * seg_elems * 4
             dst.append(recv[r].data_ptr() + off)
             a.append(send[r].data_ptr() + off)
-            b.append(send[(r + 1) % world].data_ptr() + off)
+            b.append(recv[(r + world // 2) % world].data_ptr() + off)
         shapes.append(((vp * k)(*dst), (vp * k)(*a), (vp * k)(*b), (C.c_size_t * k)(*([seg_elems] * k))))
     L = H.lib()
 
@@ -136,8 +143,8 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
-        "traffic": None,
-        "kernel": "ibcomm_hip::SegmentKernel<float, f32x4, 256, 1, true>",
+        "traffic": MEASURED_TRAFFIC_BYTES.get("%d segments x %d fp32" % (k, seg_elems)),
+        "kernel": "ibcomm_hip::SegmentKernel<float, float4, 256, 1, nontemporal, add>",
         "launch_shape": "%d segments x %d fp32" % (k, seg_elems),
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
@@ -184,6 +191,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="issue every step eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
+    ap.add_argument("--only-roofline", action="store_true",
+                    help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -209,6 +218,23 @@ def main():
     recv = [torch.empty_like(t) for t in send]
     sp = [t.data_ptr() for t in send]
     rp = [t.data_ptr() for t in recv]
+
+    if args.only_roofline:
+        p = H.Plan(algo, world, 0, n, 4, chunk)
+        fuse = args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64"))
+        if algo == H.RING:
+            per_step = len(p.ranges) // world            # one ring step reduces one group
+        else:
+            per_step = sum(1 for _, peer, kind in p.recvs if kind == 0)  # the first halving step's window
+        seg_elems = p.ranges[0][1] - p.ranges[0][0]
+        # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
+        # counters collected over this command can be calibrated against a known traffic
+        for _ in range(3):
+            recv[0].copy_(send[0])
+        torch.cuda.synchronize()
+        print(json.dumps({"only_roofline": True, "config": args.config,
+                          "roofline": roofline_leg(torch, H, send, recv, seg_elems, max(1, min(fuse, per_step)), 200)}))
+        return
 
     with H.World(world) as w:
         if args.landing:
