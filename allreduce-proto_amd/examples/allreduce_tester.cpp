@@ -30,82 +30,116 @@ struct Vars {
   double p, np, n, nb, i;
 };
 
+// An expression compiled once into a postfix program and evaluated per element on a small stack.
 class Expr {
  public:
-  explicit Expr(const std::string& text) : s_(text) {}
-  bool Eval(const Vars& v, double* out) {
-    v_ = &v;
-    pos_ = 0;
-    ok_ = true;
-    const double r = Sum();
+  explicit Expr(const std::string& text) : s_(text) {
+    Sum();
     Skip();
     if (pos_ != s_.size()) ok_ = false;
-    *out = r;
-    return ok_;
+  }
+  bool ok() const { return ok_; }
+  double Eval(const Vars& v) const {
+    double st[64];
+    int top = 0;
+    for (const Ins& in : prog_) {
+      switch (in.op) {
+        case kNum: st[top++] = in.value; break;
+        case kP: st[top++] = v.p; break;
+        case kNp: st[top++] = v.np; break;
+        case kN: st[top++] = v.n; break;
+        case kNb: st[top++] = v.nb; break;
+        case kI: st[top++] = v.i; break;
+        case kNeg: st[top - 1] = -st[top - 1]; break;
+        case kAdd: top--; st[top - 1] += st[top]; break;
+        case kSub: top--; st[top - 1] -= st[top]; break;
+        case kMul: top--; st[top - 1] *= st[top]; break;
+        case kDiv: top--; st[top - 1] /= st[top]; break;
+      }
+    }
+    return top == 1 ? st[0] : 0.0;
   }
 
  private:
+  enum Op { kNum, kP, kNp, kN, kNb, kI, kNeg, kAdd, kSub, kMul, kDiv };
+  struct Ins {
+    Op op;
+    double value;
+  };
+  void Emit(Op op, double value = 0) {
+    prog_.push_back(Ins{op, value});
+    if (op <= kI) {
+      if (++depth_ > 60) ok_ = false;
+    } else if (op != kNeg) {
+      depth_--;
+    }
+  }
   void Skip() {
     while (pos_ < s_.size() && isspace(static_cast<unsigned char>(s_[pos_]))) pos_++;
   }
-  double Sum() {
-    double a = Product();
+  bool Eat(char c) {
+    Skip();
+    if (pos_ < s_.size() && s_[pos_] == c) {
+      pos_++;
+      return true;
+    }
+    return false;
+  }
+  void Sum() {
+    Product();
     for (;;) {
-      Skip();
-      if (pos_ < s_.size() && s_[pos_] == '+') { pos_++; a += Product(); }
-      else if (pos_ < s_.size() && s_[pos_] == '-') { pos_++; a -= Product(); }
-      else return a;
+      if (Eat('+')) { Product(); Emit(kAdd); }
+      else if (Eat('-')) { Product(); Emit(kSub); }
+      else return;
     }
   }
-  double Product() {
-    double a = Unary();
+  void Product() {
+    Unary();
     for (;;) {
-      Skip();
-      if (pos_ < s_.size() && s_[pos_] == '*') { pos_++; a *= Unary(); }
-      else if (pos_ < s_.size() && s_[pos_] == '/') { pos_++; a /= Unary(); }
-      else return a;
+      if (Eat('*')) { Unary(); Emit(kMul); }
+      else if (Eat('/')) { Unary(); Emit(kDiv); }
+      else return;
     }
   }
-  double Unary() {
-    Skip();
-    if (pos_ < s_.size() && s_[pos_] == '-') { pos_++; return -Unary(); }
-    if (pos_ < s_.size() && s_[pos_] == '+') { pos_++; return Unary(); }
-    return Atom();
+  void Unary() {
+    if (Eat('-')) { Unary(); Emit(kNeg); return; }
+    if (Eat('+')) { Unary(); return; }
+    Atom();
   }
-  double Atom() {
+  void Atom() {
     Skip();
-    if (pos_ >= s_.size()) { ok_ = false; return 0; }
+    if (pos_ >= s_.size()) { ok_ = false; Emit(kNum, 0); return; }
     if (s_[pos_] == '(') {
       pos_++;
-      const double a = Sum();
-      Skip();
-      if (pos_ < s_.size() && s_[pos_] == ')') pos_++;
-      else ok_ = false;
-      return a;
+      Sum();
+      if (!Eat(')')) ok_ = false;
+      return;
     }
     if (isdigit(static_cast<unsigned char>(s_[pos_])) || s_[pos_] == '.') {
       char* end = nullptr;
       const double a = strtod(s_.c_str() + pos_, &end);
       pos_ = static_cast<size_t>(end - s_.c_str());
-      return a;
+      Emit(kNum, a);
+      return;
     }
     if (isalpha(static_cast<unsigned char>(s_[pos_]))) {
-      size_t b = pos_;
+      const size_t b = pos_;
       while (pos_ < s_.size() && isalnum(static_cast<unsigned char>(s_[pos_]))) pos_++;
       const std::string name = s_.substr(b, pos_ - b);
-      if (name == "p") return v_->p;
-      if (name == "np") return v_->np;
-      if (name == "n") return v_->n;
-      if (name == "nb") return v_->nb;
-      if (name == "i") return v_->i;
+      if (name == "p") return Emit(kP);
+      if (name == "np") return Emit(kNp);
+      if (name == "n") return Emit(kN);
+      if (name == "nb") return Emit(kNb);
+      if (name == "i") return Emit(kI);
     }
     ok_ = false;
-    return 0;
+    Emit(kNum, 0);
   }
   std::string s_;
   size_t pos_ = 0;
   bool ok_ = true;
-  const Vars* v_ = nullptr;
+  int depth_ = 0;
+  std::vector<Ins> prog_;
 };
 
 bool ParseBytes(const char* src, size_t* out) {  // allreduce_tester.cpp:205-238
@@ -128,7 +162,7 @@ bool ParseBytes(const char* src, size_t* out) {  // allreduce_tester.cpp:205-238
     hipError_t e_ = (cmd);                                                                     \
     if (e_ != hipSuccess) {                                                                    \
       fprintf(stderr, "%s failed: %s\n", #cmd, hipGetErrorString(e_));                         \
-      exit(static_cast<int>(util::IBCOMM_ERROR_CODE::CUDA_ERROR));                             \
+      util::EndProcess(util::IBCOMM_ERROR_CODE::CUDA_ERROR);                                   \
     }                                                                                          \
   } while (0)
 
@@ -156,6 +190,12 @@ int main(int argc, char** argv) {
   }
   const size_t n = nbytes / sizeof(ElemType);
   const std::string init_expr = argv[4], check_expr = argv[5];
+  for (const std::string& e : {init_expr, check_expr}) {
+    if (!Expr(e).ok()) {
+      fprintf(stderr, "Invalid expression: '%s'\n", e.c_str());
+      return 1;
+    }
+  }
 
   HIP_OR_EXIT(hipSetDevice(0));
   std::vector<std::unique_ptr<IBVerbsCommunicator>> comms;
@@ -174,12 +214,10 @@ int main(int argc, char** argv) {
     threads.emplace_back([&, r]() {
       Vars v{static_cast<double>(r), static_cast<double>(np), static_cast<double>(n), static_cast<double>(nbytes), 0};
       std::vector<ElemType> host(n);
-      Expr init(init_expr);
+      const Expr init(init_expr);
       for (size_t i = 0; i < n; i++) {
         v.i = static_cast<double>(i);
-        double x;
-        if (!init.Eval(v, &x)) { fprintf(stderr, "Invalid expression: '%s'\n", init_expr.c_str()); exit(1); }
-        host[i] = static_cast<ElemType>(x);
+        host[i] = static_cast<ElemType>(init.Eval(v));
       }
       ElemType *send = nullptr, *recv = nullptr;
       HIP_OR_EXIT(hipMalloc(&send, n * sizeof(ElemType)));
@@ -188,12 +226,11 @@ int main(int argc, char** argv) {
       if (algorithm == "ring") comms[r]->AllreduceRingCuda(send, recv, n);
       else comms[r]->AllreduceRabenseifnerCuda(send, recv, n);
       HIP_OR_EXIT(hipMemcpy(host.data(), recv, n * sizeof(ElemType), hipMemcpyDeviceToHost));
-      Expr check(check_expr);
+      const Expr check(check_expr);
       size_t reported = 0;
       for (size_t i = 0; i < n; i++) {
         v.i = static_cast<double>(i);
-        double want;
-        if (!check.Eval(v, &want)) { fprintf(stderr, "Invalid expression: '%s'\n", check_expr.c_str()); exit(1); }
+        const double want = check.Eval(v);
         if (std::fabs(static_cast<double>(host[i]) - want) > 1e-12) {
           failed[r] = 1;
           if (reported++ < 10) fprintf(stderr, "[Rank %d] Error: Element [%zu] must be %g but actually is %d\n", r, i, want, host[i]);

@@ -5,6 +5,8 @@
 #include <cstdio>
 #include <cstdlib>
 
+#include <unistd.h>
+
 namespace util {
 
 enum class IBCOMM_ERROR_CODE : int {
@@ -15,10 +17,18 @@ enum class IBCOMM_ERROR_CODE : int {
 };
 
 // Prints where and why, then ends the process with the error code as exit status: callers of the
-// reference (and its tests, tests/allreduce_test.py:95-97) rely on that exit status.
+// reference (and its tests, tests/allreduce_test.py:95-97) rely on that exit status.  Several
+// emulated ranks of one process usually hit the same error at the same moment, and exit() must not
+// run its handlers on two threads at once, so the process ends with _exit() after flushing.
+[[noreturn]] inline void EndProcess(IBCOMM_ERROR_CODE error_code) {
+  fflush(stdout);
+  fflush(stderr);
+  _exit(static_cast<int>(error_code));
+}
+
 [[noreturn]] inline void IbcommError(const char* filename, int line, IBCOMM_ERROR_CODE error_code, const char* message) {
   fprintf(stderr, "Error occured at %s:L%d.\n%s\n", filename, line, message);
-  exit(static_cast<int>(error_code));
+  EndProcess(error_code);
 }
 
 template <typename A, typename... Args>
@@ -27,7 +37,7 @@ template <typename A, typename... Args>
   fprintf(stderr, "Error occured at %s:L%d.\n", filename, line);
   fprintf(stderr, format, a, args...);
   fputs("\n", stderr);
-  exit(static_cast<int>(error_code));
+  EndProcess(error_code);
 }
 
 inline void IbcommWarning(const char* filename, int line, const char* message) {

@@ -77,7 +77,8 @@ def test_a_wrong_answer_is_reported_in_the_exit_status():
 
 @pytest.mark.slow
 def test_aging():
-    for _ in range(10):
+    # the reference repeats each 100 times (tests/allreduce_test.py:227-235); a few keep the suite short
+    for _ in range(3):
         assert check(algo=ALGO_RING, np=4, buffsize="128M") == 0
-    for _ in range(10):
+    for _ in range(3):
         assert check(algo=ALGO_RABEN, np=4, buffsize="128M") == 0
