@@ -71,9 +71,20 @@ struct HipBackend {
     IBCOMM_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
     return kOk;
   }
-  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s) {
-    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, DefaultTuning(), s));
+  // `role` says what the launch is for, so that each can carry its own cache hints:
+  // 0 = reduction, 1 = landing copy into a pool slot, 2 = gather into recvbuf.
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int role = 0) {
+    LaunchTuning t = DefaultTuning();
+    static const int nt_reduce = EnvMask("IBCOMM_HIP_NT_REDUCE", t.nontemporal);
+    static const int nt_landing = EnvMask("IBCOMM_HIP_NT_LANDING", t.nontemporal);
+    static const int nt_gather = EnvMask("IBCOMM_HIP_NT_GATHER", t.nontemporal);
+    t.nontemporal = role == 0 ? nt_reduce : (role == 1 ? nt_landing : nt_gather);
+    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, t, s));
     return kOk;
+  }
+  static int EnvMask(const char* name, int fallback) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : fallback;
   }
 };
 

@@ -22,13 +22,14 @@ static_assert(IBCOMM_HIP_RING == kRing && IBCOMM_HIP_RABENSEIFNER == kRabenseifn
 // length, chunk size and knobs, so the sequence is captured once and replayed: the host then costs
 // one hipGraphLaunch instead of hundreds of launches and event calls per collective.
 struct GraphKey {
-  int algo = 0, dtype = 0, landing = 0, fuse = 0, world = 0;
+  int algo = 0, dtype = 0, landing = 0, fuse = 0, world = 0, replay_rank = -1;
   size_t len = 0;
   std::string chunk_env;
   std::vector<const void*> send;
   std::vector<void*> recv;
   bool operator==(const GraphKey& o) const {
-    return algo == o.algo && dtype == o.dtype && landing == o.landing && fuse == o.fuse && world == o.world && len == o.len &&
+    return algo == o.algo && dtype == o.dtype && landing == o.landing && fuse == o.fuse && world == o.world &&
+           replay_rank == o.replay_rank && len == o.len &&
            chunk_env == o.chunk_env && send == o.send && recv == o.recv;
   }
 };
@@ -151,6 +152,8 @@ int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* c, const int32_t* s, 
   return ibcomm_hip_allreduce_rabenseifner(c, kI32, s, r, n);
 }
 
+}  // extern "C"
+
 namespace {
 
 constexpr size_t kMaxCachedGraphs = 16;
@@ -170,8 +173,9 @@ int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g) {
 // the ranks' own multi-stream, event-linked work gave graphs whose instantiation did not finish.
 // Launches at the default fusion are large enough to fill the GPU on their own, so the chain costs
 // little overlap and removes the host's launch and event work from every later call.
-int CaptureWorld(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key,
-                 const void* const* sendbufs, void* const* recvbufs, CachedGraph* out) {
+template <class IssueFn>
+int CaptureIssue(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key, IssueFn issue,
+                 CachedGraph* out) {
   if (!f->origin) IBCOMM_HIP_CHECK(hipStreamCreateWithFlags(&f->origin, hipStreamNonBlocking));
   for (auto* c : cs) c->pool().OverrideStream(f->origin);
   hipError_t e = hipStreamBeginCapture(f->origin, hipStreamCaptureModeRelaxed);
@@ -179,7 +183,7 @@ int CaptureWorld(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& c
   if (e != hipSuccess) {
     rc = Fail(kDeviceError, "hipStreamBeginCapture failed: %s", hipGetErrorString(e));
   } else {
-    rc = RunWorld<HipBackend>(cs.data(), key.world, key.algo, key.dtype, sendbufs, recvbufs, key.len, false);
+    rc = issue(false);
   }
   for (auto* c : cs) c->pool().ClearOverride();
   if (e != hipSuccess) return rc;
@@ -203,46 +207,21 @@ int CaptureWorld(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& c
   return kOk;
 }
 
-}  // namespace
-
-int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
-                               const void* const* sendbufs, void* const* recvbufs, size_t len) {
-  if (!comms || !sendbufs || !recvbufs || world_size < 1) return Fail(kInvalidArgument, "null argument");
-  std::vector<Communicator<HipBackend>*> cs(world_size);
-  for (int r = 0; r < world_size; r++) {
-    if (!comms[r]) return Fail(kInvalidArgument, "comms[%d] is null", r);
-    if (comms[r]->owner != comms[0]->owner) return Fail(kInvalidArgument, "communicators belong to different fabrics");
-    cs[r] = &comms[r]->comm;
-  }
-  ibcomm_hip_fabric* f = comms[0]->owner;
-  // Recording hipMemcpyAsync device-to-device copies into a graph crashed the host process inside
-  // the runtime on ROCm 7.2 (gfx950), so the per-message-memcpy landing mode is never recorded.
-  if (f->graph_mode == 0 || world_size == 1 || cs[0]->landing() == kLandMemcpy) {
+// Eager on the first use of a call shape, recorded on the second, replayed from then on.
+// `issue(synchronize)` issues the device work of one call on the communicators in `cs`.
+template <class IssueFn>
+int IssueCached(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key, bool may_record,
+                IssueFn issue) {
+  if (!may_record) {
     f->eager_calls++;
-    return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+    return issue(true);
   }
-
-  GraphKey key;
-  key.algo = algo;
-  key.dtype = dtype;
-  key.landing = cs[0]->landing();
-  key.fuse = cs[0]->max_fuse();
-  key.world = world_size;
-  key.len = len;
-  const char* env = getenv("IBCOMM_CHUNKSIZE");  // read on every call, like the reference
-  key.chunk_env = env ? env : "";
-  key.send.assign(sendbufs, sendbufs + world_size);
-  key.recv.assign(recvbufs, recvbufs + world_size);
-  for (int r = 1; r < world_size; r++)
-    if (cs[r]->landing() != key.landing || cs[r]->max_fuse() != key.fuse) key.fuse = -1 - r;  // mixed knobs: never equal
-
   for (CachedGraph& g : f->graphs)
     if (g.key == key) return ReplayGraph(f, g);
 
   if (f->has_last_eager && f->last_eager == key) {
-    // Second call with this shape: record it.  The recording itself executes nothing, so launch it once.
     CachedGraph g;
-    const int rc = CaptureWorld(f, cs, key, sendbufs, recvbufs, &g);
+    const int rc = CaptureIssue(f, cs, key, issue, &g);
     if (rc != kOk) {
       for (auto* c : cs) c->Abort();
       f->fabric.Reset();
@@ -256,17 +235,101 @@ int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, in
       f->graphs.erase(f->graphs.begin());
     }
     f->graphs.push_back(g);
-    return ReplayGraph(f, f->graphs.back());
+    return ReplayGraph(f, f->graphs.back());  // recording executes nothing: run it once
   }
 
   f->eager_calls++;
   uint64_t ops_before = 0, ops_after = 0;
   for (auto* c : cs) ops_before += DeviceOps(c->stats());
-  const int rc = RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+  const int rc = issue(true);
   for (auto* c : cs) ops_after += DeviceOps(c->stats());
   // Only shapes of a bounded number of device operations are recorded on their next use.
   f->has_last_eager = (rc == kOk) && (ops_after - ops_before <= f->graph_max_ops);
   if (rc == kOk) f->last_eager = key;
+  return rc;
+}
+
+GraphKey MakeKey(std::vector<Communicator<HipBackend>*>& cs, int algo, int dtype, size_t len, const void* const* sendbufs,
+                 void* const* recvbufs, int replay_rank) {
+  GraphKey key;
+  key.algo = algo;
+  key.dtype = dtype;
+  key.landing = cs[0]->landing();
+  key.fuse = cs[0]->max_fuse();
+  key.world = cs[0]->world_size();
+  key.replay_rank = replay_rank;
+  key.len = len;
+  const char* env = getenv("IBCOMM_CHUNKSIZE");  // read on every call, like the reference
+  key.chunk_env = env ? env : "";
+  key.send.assign(sendbufs, sendbufs + cs.size());
+  key.recv.assign(recvbufs, recvbufs + cs.size());
+  for (size_t r = 1; r < cs.size(); r++)
+    if (cs[r]->landing() != key.landing || cs[r]->max_fuse() != key.fuse) key.fuse = -1 - static_cast<int>(r);  // mixed knobs: never equal
+  return key;
+}
+
+int CollectWorld(ibcomm_hip_comm* const* comms, int world_size, std::vector<Communicator<HipBackend>*>* cs) {
+  cs->resize(world_size);
+  for (int r = 0; r < world_size; r++) {
+    if (!comms[r]) return Fail(kInvalidArgument, "comms[%d] is null", r);
+    if (comms[r]->owner != comms[0]->owner) return Fail(kInvalidArgument, "communicators belong to different fabrics");
+    (*cs)[r] = &comms[r]->comm;
+  }
+  return kOk;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
+                               const void* const* sendbufs, void* const* recvbufs, size_t len) {
+  if (!comms || !sendbufs || !recvbufs || world_size < 1) return Fail(kInvalidArgument, "null argument");
+  std::vector<Communicator<HipBackend>*> cs;
+  IBCOMM_RETURN_IF_ERROR(CollectWorld(comms, world_size, &cs));
+  ibcomm_hip_fabric* f = comms[0]->owner;
+  // Recording hipMemcpyAsync device-to-device copies into a graph crashed the host process inside
+  // the runtime on ROCm 7.2 (gfx950), so the per-message-memcpy landing mode is never recorded.
+  const bool may_record = f->graph_mode != 0 && world_size > 1 && cs[0]->landing() != kLandMemcpy;
+  const GraphKey key = MakeKey(cs, algo, dtype, len, sendbufs, recvbufs, -1);
+  return IssueCached(f, cs, key, may_record, [&](bool synchronize) {
+    return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, synchronize);
+  });
+}
+
+int ibcomm_hip_world_record(ibcomm_hip_comm* const* comms, int world_size, int rank, int algo, int dtype,
+                            const void* const* sendbufs, void* const* recvbufs, size_t len) {
+  if (!comms || !sendbufs || !recvbufs || world_size < 2) return Fail(kInvalidArgument, "recording needs a world of at least 2");
+  if (rank < 0 || rank >= world_size) return Fail(kInvalidArgument, "rank %d outside world of %d", rank, world_size);
+  std::vector<Communicator<HipBackend>*> cs;
+  IBCOMM_RETURN_IF_ERROR(CollectWorld(comms, world_size, &cs));
+  ibcomm_hip_fabric* f = comms[0]->owner;
+  size_t log_bytes = 0;
+  IBCOMM_RETURN_IF_ERROR(cs[rank]->RecordingBytes(algo, dtype, len, &log_bytes));
+  f->DropGraphs();  // replay graphs point into the log, which is about to be rewritten (and may move)
+  f->has_last_eager = false;
+  IBCOMM_RETURN_IF_ERROR(f->fabric.StartRecording(rank, log_bytes));
+  f->eager_calls++;
+  const int rc = RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
+  f->fabric.StopRecording();
+  return rc;
+}
+
+int ibcomm_hip_replay_allreduce(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  ibcomm_hip_fabric* f = comm->owner;
+  const int rank = comm->comm.rank();
+  if (!f->fabric.StartReplay(rank))
+    return Fail(kInvalidArgument, "no recording for rank %d: call ibcomm_hip_world_record first", rank);
+  std::vector<Communicator<HipBackend>*> cs(1, &comm->comm);
+  const void* sends[1] = {sendbuf};
+  void* recvs[1] = {recvbuf};
+  const bool may_record = f->graph_mode != 0 && comm->comm.landing() != kLandMemcpy;
+  const GraphKey key = MakeKey(cs, algo, dtype, len, sends, recvs, rank);
+  const int rc = IssueCached(f, cs, key, may_record, [&](bool synchronize) {
+    return RunAlone<HipBackend>(&comm->comm, algo, dtype, sendbuf, recvbuf, len, synchronize);
+  });
+  f->fabric.StopReplay();
   return rc;
 }
 

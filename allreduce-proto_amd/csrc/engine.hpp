@@ -269,6 +269,18 @@ class Communicator {
     return Finish(true);
   }
 
+  // Bytes of log a recording of this rank's side of the given collective needs.
+  int RecordingBytes(int algo, int dtype, size_t len_elements, size_t* out) {
+    Plan p;
+    const size_t es = DTypeSize(dtype);
+    if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+    IBCOMM_RETURN_IF_ERROR(BuildPlan(algo, world_size_, rank_, len_elements, es, getenv("IBCOMM_CHUNKSIZE"), &p));
+    size_t total = 0;
+    for (const RecvOp& r : p.recvs) total += (p.part.ranges[r.chunk].size() * es + 255) & ~size_t(255);
+    *out = total;
+    return kOk;
+  }
+
   const Plan& plan() const { return plan_; }
   bool active() const { return active_; }
   size_t recv_cursor() const { return next_recv_; }
@@ -393,7 +405,7 @@ class Communicator {
       // A gather overwrites recvbuf[chunk]; a send of ours out of that range must have been read first.
       if (r.kind == kGather && chunk_unconsumed_[r.chunk] > 0) break;
       PendingRecv p;
-      if (!fabric_->Take(rank_, r.peer, &p.msg)) break;
+      if (!fabric_->Take(rank_, r.peer, &p.msg, next_send_)) break;
       if (p.msg.bytes != ChunkBytes(r.chunk))
         return Fail(kTransportError, "rank %d: message of %zu bytes from rank %d where chunk %d has %zu", rank_, p.msg.bytes,
                     r.peer, r.chunk, ChunkBytes(r.chunk));
@@ -434,10 +446,11 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
+        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
         batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, p.msg.src, nullptr, ChunkElems(c)};
         stats_.gather_bytes += ChunkBytes(c);
       }
-      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s));
+      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 2));
       stats_.gather_copies++;
       OpState done;
       IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
@@ -456,6 +469,7 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
+        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
         IBCOMM_RETURN_IF_ERROR(B::CopyAsync(RecvPtr(c), p.msg.src, ChunkBytes(c), s));
         stats_.gather_copies++;
         stats_.gather_bytes += ChunkBytes(c);
@@ -485,6 +499,7 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&si));
         IBCOMM_RETURN_IF_ERROR(WaitOnMessage(si, p.msg));
         IBCOMM_RETURN_IF_ERROR(WaitOnSlot(si, p.slot));
+        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, si));
         IBCOMM_RETURN_IF_ERROR(B::CopyAsync(p.slot->LandingFor(RecvPtr(r.chunk)), p.msg.src, ChunkBytes(r.chunk), si));
         stats_.landing_copies++;
         stats_.landing_bytes += ChunkBytes(r.chunk);
@@ -495,7 +510,10 @@ class Communicator {
       for (size_t i = 1; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOn(s, landed[i]));
     } else {
       IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
-      for (size_t i = 0; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, pending_reduce_[i].msg));
+      for (size_t i = 0; i < n; i++) {
+        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, pending_reduce_[i].msg));
+        IBCOMM_RETURN_IF_ERROR(RecordPayload(pending_reduce_[i].msg, s));
+      }
       if (landing_ == kLandKernel) {
         SegmentBatch copy;
         copy.count = 0;
@@ -506,7 +524,7 @@ class Communicator {
           copy.seg[copy.count++] = Segment{p.slot->LandingFor(RecvPtr(c)), nullptr, p.msg.src, nullptr, ChunkElems(c)};
           stats_.landing_bytes += ChunkBytes(c);
         }
-        IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s));
+        IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
         stats_.landing_copies++;
         OpState done;
         IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
@@ -534,7 +552,7 @@ class Communicator {
       batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, incoming, own, ChunkElems(c)};
       stats_.reduce_elements += ChunkElems(c);
     }
-    IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s));
+    IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 0));
     stats_.reduce_launches++;
     stats_.reduce_segments += n;
     OpState done;
@@ -550,6 +568,12 @@ class Communicator {
     }
     pending_reduce_.clear();
     return kOk;
+  }
+
+  // While this rank's traffic is being recorded for replay, keep a copy of the message's payload.
+  int RecordPayload(const Message& m, Stream s) {
+    if (!m.record_to) return kOk;
+    return B::CopyAsync(m.record_to, m.src, m.bytes, s);
   }
 
   int WaitOnSlot(Stream s, const Memory<B>* slot) {

@@ -42,6 +42,7 @@ class Fabric {
     bool has_ready = false;
     typename B::Stream ready_stream{};  // stream `ready` was recorded on (a wait from that same stream is redundant)
     uint64_t ticket = 0;
+    char* record_to = nullptr;          // while recording: where the receiver must also copy the payload
   };
   struct Completion {
     uint64_t ticket = 0;
@@ -60,6 +61,13 @@ class Fabric {
                     typename B::Stream ready_stream = typename B::Stream{}) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
+    if (from == replay_rank_) {
+      // The peer is a ghost: nobody will read the data, the send is complete at once.
+      Completion k;
+      k.ticket = c.next_ticket++;
+      c.completions.push_back(k);
+      return k.ticket;
+    }
     Message m;
     m.src = src;
     m.bytes = bytes;
@@ -74,13 +82,29 @@ class Fabric {
 
   // Receiver: remove and return the oldest message `from` has posted for `to`.  The receiver now
   // owes exactly one Complete() for it, and must complete a channel's messages in the order taken.
-  bool Take(int to, int from, Message* out) {
+  // `sends_posted` is how many messages the receiver itself has emitted so far in this collective;
+  // it only matters for recording and replay (below).
+  bool Take(int to, int from, Message* out, size_t sends_posted = 0) {
+    if (to == replay_rank_) return GhostTake(from, out, sends_posted);
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
     if (c.inbox.empty() || c.inbox.front().ticket >= c.visible_below) return false;
     *out = c.inbox.front();
     c.inbox.pop_front();
     c.taken++;
+    if (to == record_rank_) {
+      // Remember the message for replay: its size, its sender, and how far the receiver had got with
+      // its own sends when the message was there to take.  The receiver copies the payload to
+      // out->record_to (a range of the log) when it lands the message.
+      LogEntry e;
+      e.from = from;
+      e.bytes = out->bytes;
+      e.gate = sends_posted;
+      e.offset = log_used_;
+      log_used_ += (out->bytes + 255) & ~size_t(255);
+      out->record_to = log_used_ <= log_bytes_ ? log_base_ + e.offset : nullptr;
+      log_.push_back(e);
+    }
     return true;
   }
 
@@ -105,6 +129,7 @@ class Fabric {
   // Receiver: the pull of message `ticket` has been enqueued; `done` completes when it has read the source.
   void Complete(int to, int from, uint64_t ticket, typename B::Event done, bool has_done,
                 typename B::Stream done_stream = typename B::Stream{}) {
+    if (to == replay_rank_) return;  // recorded messages have no sender waiting for them
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
     Completion k;
@@ -143,6 +168,67 @@ class Fabric {
     return t;
   }
 
+  // ---- recording one rank's incoming traffic, and replaying it -------------------------------
+  //
+  // Measuring one rank's share of a collective needs that rank to run alone, yet every message it
+  // consumes is a partial sum produced by the others.  So one ordinary run of the whole world is
+  // recorded: each message `rank` takes is copied into a device-resident log together with the
+  // number of sends `rank` had posted when the message was available.  In a replay the other ranks
+  // are ghosts: `rank` finds the logged messages in its channels, each visible once it has itself
+  // posted as many sends as it had in the recorded run (which paces the replay the way the real
+  // dependency on upstream ranks does), and its own sends complete immediately.
+
+  // Arms recording for the next collective.  log_bytes must cover the payload of every message
+  // `rank` will take (each rounded up to 256 bytes).
+  int StartRecording(int rank, size_t log_bytes) {
+    StopReplay();
+    if (log_base_ && log_bytes_ < log_bytes) {
+      B::Free(log_base_);
+      log_base_ = nullptr;
+    }
+    if (!log_base_) {
+      void* p = nullptr;
+      const int rc = B::Malloc(&p, log_bytes);
+      if (rc != 0) return rc;
+      log_base_ = static_cast<char*>(p);
+      log_bytes_ = log_bytes;
+    }
+    log_.clear();
+    log_used_ = 0;
+    record_rank_ = rank;
+    recorded_rank_ = -1;
+    return 0;
+  }
+  // Ends recording; the log now describes `rank`'s side of the collective just run.
+  void StopRecording() {
+    if (record_rank_ >= 0 && log_used_ <= log_bytes_) recorded_rank_ = record_rank_;
+    record_rank_ = -1;
+  }
+  int recording_rank() const { return record_rank_; }
+  int recorded_rank() const { return recorded_rank_; }
+  size_t recorded_messages() const { return log_.size(); }
+
+  // From now on `rank` runs alone against the recorded messages.  False if nothing was recorded for it.
+  bool StartReplay(int rank) {
+    if (recorded_rank_ != rank) return false;
+    replay_rank_ = rank;
+    RewindReplay();
+    return true;
+  }
+  void RewindReplay() { log_cursor_ = 0; }
+  void StopReplay() { replay_rank_ = -1; }
+  int replay_rank() const { return replay_rank_; }
+  bool ReplayDrained() const { return log_cursor_ == log_.size(); }
+
+  void FreeLog() {
+    if (log_base_) B::Free(log_base_);
+    log_base_ = nullptr;
+    log_bytes_ = 0;
+    log_.clear();
+    recorded_rank_ = -1;
+  }
+  ~Fabric() { FreeLog(); }
+
   // Drops everything queued; used when a collective is abandoned after an error.
   void Reset() {
     for (auto& c : channels_) {
@@ -153,6 +239,25 @@ class Fabric {
   }
 
  private:
+  struct LogEntry {
+    int from;
+    size_t bytes;
+    size_t gate;    // sends the recorded rank had posted when this message was available
+    size_t offset;  // of the payload in the log
+  };
+
+  bool GhostTake(int from, Message* out, size_t sends_posted) {
+    if (log_cursor_ >= log_.size()) return false;
+    const LogEntry& e = log_[log_cursor_];
+    if (e.from != from || sends_posted < e.gate) return false;
+    *out = Message();
+    out->src = log_base_ + e.offset;
+    out->bytes = e.bytes;
+    out->ticket = log_cursor_;
+    log_cursor_++;
+    return true;
+  }
+
   struct Channel {
     std::mutex mu;
     std::deque<Message> inbox;
@@ -167,6 +272,12 @@ class Fabric {
 
   int n_;
   std::vector<std::unique_ptr<Channel>> channels_;
+  int record_rank_ = -1;    // rank whose incoming messages are being logged
+  int recorded_rank_ = -1;  // rank the finished log belongs to
+  int replay_rank_ = -1;    // rank currently running against the log
+  char* log_base_ = nullptr;
+  size_t log_bytes_ = 0, log_used_ = 0, log_cursor_ = 0;
+  std::vector<LogEntry> log_;
 };
 
 }  // namespace ibcomm_hip

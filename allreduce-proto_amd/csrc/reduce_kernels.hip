@@ -27,7 +27,9 @@ __device__ __forceinline__ void StoreVec(V* p, V v) {
 // vector of T.  Integer types are instantiated unsigned so that += wraps.
 // ADD selects dst = a + b; otherwise the launch is a copy, dst = a.  The two are
 // separate kernels so that a profile tells reductions from landing copies.
-template <typename T, typename V, int THREADS, int UNROLL, bool NT, bool ADD>
+// NT is a mask of which accesses carry the non-temporal hint: 1 = loads of a,
+// 2 = loads of b, 4 = stores.
+template <typename T, typename V, int THREADS, int UNROLL, int NT, bool ADD>
 __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batch) {
   const Segment s = batch.seg[blockIdx.y];
   const uint64_t n = s.n;
@@ -67,28 +69,28 @@ __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batc
       V rb[UNROLL];
       if (base + kTile <= nvec) {
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) ra[u] = LoadVec<NT>(av + base + u * THREADS + threadIdx.x);
+        for (int u = 0; u < UNROLL; u++) ra[u] = LoadVec<(NT & 1) != 0>(av + base + u * THREADS + threadIdx.x);
         if (has_b) {
 #pragma unroll
-          for (int u = 0; u < UNROLL; u++) rb[u] = LoadVec<NT>(bv + base + u * THREADS + threadIdx.x);
+          for (int u = 0; u < UNROLL; u++) rb[u] = LoadVec<(NT & 2) != 0>(bv + base + u * THREADS + threadIdx.x);
 #pragma unroll
           for (int u = 0; u < UNROLL; u++) ra[u] = ra[u] + rb[u];
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) StoreVec<NT>(dv + base + u * THREADS + threadIdx.x, ra[u]);
+        for (int u = 0; u < UNROLL; u++) StoreVec<(NT & 4) != 0>(dv + base + u * THREADS + threadIdx.x, ra[u]);
         if (has_d2) {
 #pragma unroll
-          for (int u = 0; u < UNROLL; u++) StoreVec<NT>(d2v + base + u * THREADS + threadIdx.x, ra[u]);
+          for (int u = 0; u < UNROLL; u++) StoreVec<(NT & 4) != 0>(d2v + base + u * THREADS + threadIdx.x, ra[u]);
         }
       } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
           const uint64_t i = base + u * THREADS + threadIdx.x;
           if (i < nvec) {
-            V v = LoadVec<NT>(av + i);
-            if (has_b) v = v + LoadVec<NT>(bv + i);
-            StoreVec<NT>(dv + i, v);
-            if (has_d2) StoreVec<NT>(d2v + i, v);
+            V v = LoadVec<(NT & 1) != 0>(av + i);
+            if (has_b) v = v + LoadVec<(NT & 2) != 0>(bv + i);
+            StoreVec<(NT & 4) != 0>(dv + i, v);
+            if (has_d2) StoreVec<(NT & 4) != 0>(d2v + i, v);
           }
         }
       }
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batc
 
 namespace {
 
-template <typename T, typename V, int THREADS, int UNROLL, bool NT>
+template <typename T, typename V, int THREADS, int UNROLL, int NT>
 hipError_t LaunchOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
   if (batch.seg[0].b != nullptr)
     hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, UNROLL, NT, true>), grid, dim3(THREADS), 0, stream, batch);
@@ -121,18 +123,25 @@ hipError_t LaunchOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
 }
 
 template <typename T, typename V, int THREADS, int UNROLL>
-hipError_t LaunchNT(const SegmentBatch& batch, dim3 grid, bool nt, hipStream_t stream) {
-  return nt ? LaunchOne<T, V, THREADS, UNROLL, true>(batch, grid, stream)
-            : LaunchOne<T, V, THREADS, UNROLL, false>(batch, grid, stream);
+hipError_t LaunchNT(const SegmentBatch& batch, dim3 grid, int nt, hipStream_t stream) {
+  switch (nt & 7) {
+    case 0: return LaunchOne<T, V, THREADS, UNROLL, 0>(batch, grid, stream);
+    case 1: return LaunchOne<T, V, THREADS, UNROLL, 1>(batch, grid, stream);
+    case 2: return LaunchOne<T, V, THREADS, UNROLL, 2>(batch, grid, stream);
+    case 3: return LaunchOne<T, V, THREADS, UNROLL, 3>(batch, grid, stream);
+    case 4: return LaunchOne<T, V, THREADS, UNROLL, 4>(batch, grid, stream);
+    case 5: return LaunchOne<T, V, THREADS, UNROLL, 5>(batch, grid, stream);
+    case 6: return LaunchOne<T, V, THREADS, UNROLL, 6>(batch, grid, stream);
+    default: return LaunchOne<T, V, THREADS, UNROLL, 7>(batch, grid, stream);
+  }
 }
 
 template <typename T, typename V, int THREADS>
-hipError_t LaunchUnroll(const SegmentBatch& batch, dim3 grid, int unroll, bool nt, hipStream_t stream) {
+hipError_t LaunchUnroll(const SegmentBatch& batch, dim3 grid, int unroll, int nt, hipStream_t stream) {
   switch (unroll) {
     case 1: return LaunchNT<T, V, THREADS, 1>(batch, grid, nt, stream);
     case 2: return LaunchNT<T, V, THREADS, 2>(batch, grid, nt, stream);
     case 4: return LaunchNT<T, V, THREADS, 4>(batch, grid, nt, stream);
-    case 8: return LaunchNT<T, V, THREADS, 8>(batch, grid, nt, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -141,7 +150,6 @@ template <typename T, typename V>
 hipError_t LaunchThreads(const SegmentBatch& batch, dim3 grid, const LaunchTuning& t, hipStream_t stream) {
   switch (t.threads) {
     case 256: return LaunchUnroll<T, V, 256>(batch, grid, t.unroll, t.nontemporal, stream);
-    case 512: return LaunchUnroll<T, V, 512>(batch, grid, t.unroll, t.nontemporal, stream);
     case 1024: return LaunchUnroll<T, V, 1024>(batch, grid, t.unroll, t.nontemporal, stream);
     default: return hipErrorInvalidValue;
   }
@@ -160,7 +168,7 @@ LaunchTuning DefaultTuning() {
       EnvInt("IBCOMM_HIP_THREADS", 256),
       EnvInt("IBCOMM_HIP_UNROLL", 1),
       EnvInt("IBCOMM_HIP_MAX_BLOCKS", 0),
-      EnvInt("IBCOMM_HIP_NONTEMPORAL", 1) != 0,
+      EnvInt("IBCOMM_HIP_NONTEMPORAL", 7),
   };
   return t;
 }

@@ -31,10 +31,10 @@
 namespace ibcomm_hip {
 
 struct LaunchTuning {
-  int threads;        // workgroup size: 256, 512 or 1024
-  int unroll;         // 16-byte vectors per lane per operand in flight: 1, 2, 4 or 8
+  int threads;        // workgroup size: 256 or 1024
+  int unroll;         // 16-byte vectors per lane per operand in flight: 1, 2 or 4
   int max_blocks_x;   // cap on workgroups per segment (grid-stride beyond it); 0 = no cap
-  bool nontemporal;   // stream stores (and loads) past the caches
+  int nontemporal;    // which accesses stream past the caches: 1 = loads of a, 2 = loads of b, 4 = stores
 };
 
 LaunchTuning DefaultTuning();

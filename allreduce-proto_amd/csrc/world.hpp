@@ -40,9 +40,10 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
     std::vector<char> done(n, 0);
     int remaining = n;
     Fabric<B>* fabric = comms[0]->fabric();
+    static const bool lockstep = !(getenv("IBCOMM_HIP_LOCKSTEP") && atoi(getenv("IBCOMM_HIP_LOCKSTEP")) == 0);
     while (remaining > 0 && rc == kOk) {
       bool any = false;
-      fabric->BeginSweep();
+      if (lockstep) fabric->BeginSweep();
       for (int r = 0; r < n && rc == kOk; r++) {
         if (done[r]) continue;
         bool progressed = false, finished = false;
@@ -83,6 +84,35 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
     }
   }
   return rc;
+}
+
+// One rank on its own against recorded peers (Fabric::StartReplay must be in effect for it).
+template <class B>
+int RunAlone(Communicator<B>* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len_elements,
+             bool synchronize) {
+  comm->fabric()->RewindReplay();
+  IBCOMM_RETURN_IF_ERROR(comm->Begin(algo, dtype, sendbuf, recvbuf, len_elements));
+  for (;;) {
+    bool progressed = false, finished = false;
+    const int rc = comm->Progress(&progressed, &finished);
+    if (rc != kOk) {
+      comm->Abort();
+      return rc;
+    }
+    if (finished) break;
+    if (!progressed) {
+      comm->Abort();
+      return Fail(kTransportError, "replay of rank %d stalled at receive %zu/%zu, send %zu/%zu: the recording is of a different call",
+                  comm->rank(), comm->recv_cursor(), comm->recv_total(), comm->send_cursor(), comm->send_total());
+    }
+  }
+  if (!comm->fabric()->ReplayDrained()) {
+    comm->Abort();
+    return Fail(kTransportError, "replay of rank %d left recorded messages unused: the recording is of a different call", comm->rank());
+  }
+  if (synchronize) return comm->Finish(false);
+  comm->FinishNoSync();
+  return kOk;
 }
 
 }  // namespace ibcomm_hip

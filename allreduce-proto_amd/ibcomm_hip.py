@@ -22,7 +22,7 @@ EXPORTS = [
     "ibcomm_hip_last_error", "ibcomm_hip_fabric_create", "ibcomm_hip_fabric_destroy", "ibcomm_hip_comm_create",
     "ibcomm_hip_comm_destroy", "ibcomm_hip_comm_register_myself", "ibcomm_hip_allreduce_ring",
     "ibcomm_hip_allreduce_rabenseifner", "ibcomm_hip_allreduce_ring_f32", "ibcomm_hip_allreduce_ring_i32",
-    "ibcomm_hip_allreduce_rabenseifner_f32", "ibcomm_hip_allreduce_rabenseifner_i32", "ibcomm_hip_world_allreduce",
+    "ibcomm_hip_allreduce_rabenseifner_f32", "ibcomm_hip_allreduce_rabenseifner_i32", "ibcomm_hip_world_allreduce", "ibcomm_hip_world_record", "ibcomm_hip_replay_allreduce",
     "ibcomm_hip_reduce", "ibcomm_hip_reduce_segments", "ibcomm_hip_max_segments", "ibcomm_hip_split_buffer",
     "ibcomm_hip_rank_to_chunk", "ibcomm_hip_get_exp_of_two", "ibcomm_hip_plan_create", "ibcomm_hip_plan_destroy",
     "ibcomm_hip_plan_counts", "ibcomm_hip_plan_range", "ibcomm_hip_plan_recv", "ibcomm_hip_plan_send",
@@ -62,6 +62,8 @@ def lib():
         for suffix in ("_f32", "_i32"):
             getattr(L, name + suffix).argtypes = [vp, vp, vp, sz]
     L.ibcomm_hip_world_allreduce.argtypes = [C.POINTER(vp), i, i, i, C.POINTER(vp), C.POINTER(vp), sz]
+    L.ibcomm_hip_world_record.argtypes = [C.POINTER(vp), i, i, i, i, C.POINTER(vp), C.POINTER(vp), sz]
+    L.ibcomm_hip_replay_allreduce.argtypes = [vp, i, i, vp, vp, sz]
     L.ibcomm_hip_reduce.argtypes = [i, vp, vp, vp, sz, vp]
     L.ibcomm_hip_reduce_segments.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), vp]
     L.ibcomm_hip_split_buffer.argtypes = [sz, sz, i, C.c_char_p, C.POINTER(sz), C.POINTER(sz), i, C.POINTER(i)]
@@ -179,6 +181,18 @@ class World:
         sp = (C.c_void_p * n)(*send_ptrs)
         rp = (C.c_void_p * n)(*recv_ptrs)
         return lib().ibcomm_hip_world_allreduce(comms, n, algo, dtype, sp, rp, length)
+
+    def record(self, rank, algo, dtype, send_ptrs, recv_ptrs, length):
+        """World allreduce that also records what `rank` receives, for replay()."""
+        n = self.n
+        comms = (C.c_void_p * n)(*[h.value for h in self.comms])
+        sp = (C.c_void_p * n)(*send_ptrs)
+        rp = (C.c_void_p * n)(*recv_ptrs)
+        return lib().ibcomm_hip_world_record(comms, n, rank, algo, dtype, sp, rp, length)
+
+    def replay(self, rank, algo, dtype, send_ptr, recv_ptr, length):
+        """`rank` alone against the recorded peers."""
+        return lib().ibcomm_hip_replay_allreduce(self.comms[rank], algo, dtype, send_ptr, recv_ptr, length)
 
     def allreduce_threads(self, algo, dtype, send_ptrs, recv_ptrs, length):
         """One host thread per rank, each in the blocking per-rank call (how the reference is used)."""

@@ -3,13 +3,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
 
-One "step" is one complete emulated allreduce: all N emulated ranks of the chosen BASELINE
-configuration run their whole chunk schedule on the one GPU (sendbufs resident in HBM before the
-timed region starts; every rank's recvbuf is produced).  The headline `value` is the allreduce
-algorithm bandwidth of that emulated schedule, len * 4 B / time per step, with the N ranks
-time-sharing the GPU; `extra.rank_share_algbw_GBps` is N times that (one rank's 1/N share of the
-device work).  Default workload: configs[1] of BASELINE.json (ring, 8 ranks, 256 MiB fp32 per rank,
-IBCOMM_CHUNKSIZE = 8 MiB).
+One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
+collective: every message the rank receives is landed in its HBM pool, reduced into recvbuf or
+gathered, exactly as in the full world.  The other emulated ranks are replaced by a recording of
+what they sent (made by first running the whole world once, all sendbufs resident in HBM), paced
+the way the real dependency on upstream ranks paces them.  The headline `value` is the allreduce
+algorithm bandwidth of that schedule, len * 4 B / time per step.  `extra.world_all_ranks_on_one_gpu`
+gives the same figure when all N ranks' schedules are executed on the one GPU per step.  Default
+workload: configs[1] of BASELINE.json (ring, 8 ranks, 256 MiB fp32 per rank, IBCOMM_CHUNKSIZE = 8 MiB).
 
 Two more legs, both on rank 0 of a one-GPU run:
   roofline      the dominant kernel (the segment reduction, dst = a + b at 12 B per fp32 element)
@@ -236,6 +237,18 @@ def main():
                           "roofline": roofline_leg(torch, H, send, recv, seg_elems, max(1, min(fuse, per_step)), 200)}))
         return
 
+    def timed(call, steps, warm):
+        for _ in range(warm):
+            assert call() == 0, H.last_error()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            rc = call()
+            assert rc == 0, H.last_error()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    rank = 0
     with H.World(world) as w:
         if args.landing:
             w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT}[args.landing])
@@ -243,39 +256,46 @@ def main():
             w.set_max_fuse(args.fuse)
         if args.no_graph:
             w.set_graph_mode(0)
-        # one eagerly issued step to read the per-step work counters (graph replays bypass them)
+        warm = max(args.warmup, 0 if args.no_graph else 2)  # the call shape is recorded on its second use
+
+        # 1. the whole world once, eagerly, recording what `rank` receives; its counters give the per-step work
         w.reset_stats()
-        assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0, H.last_error()
+        assert w.record(rank, algo, H.F32, sp, rp, n) == 0, H.last_error()
+        torch.cuda.synchronize()
         st = [w.stats(r) for r in range(world)]
-        # untimed: at least two more calls so that the call shape is recorded before timing starts
-        for _ in range(max(args.warmup, 0 if args.no_graph else 2)):
-            assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0, H.last_error()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            rc = w.allreduce_ptrs(algo, H.F32, sp, rp, n)
-            assert rc == 0, H.last_error()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
+        parity = check_result(torch, O, H, algo, send, recv, chunk)
+
+        # 2. THE TIMED STEP: `rank`'s complete schedule on its own, peers replaced by the recording
+        out = torch.empty_like(send[rank])
+        w.reset_stats()
+        assert w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n) == 0, H.last_error()
+        st_rank = w.stats(rank)
+        sec_per_step = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
+        parity = parity and bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
+        del out
+
+        # 3. for reference: all ranks' schedules executed on the one GPU per step
+        world_sec = timed(lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), args.steps, warm)
         graph_counters = w.graph_counters()
 
-    sec_per_step = (t1 - t0) / args.steps
-    parity = check_result(torch, O, H, algo, send, recv, chunk)
+    def device_bytes(s):
+        return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
 
-    steps = 1  # the counters in `st` cover exactly one step
-    total = {k: sum(s[k] for s in st) for k in st[0]}
-    device_bytes_per_step = (12 * total["reduce_elements"] + 2 * total["landing_bytes"] + 2 * total["gather_bytes"]) / steps
-    segs_per_launch = max(1, round(st[0]["reduce_segments"] / max(1, st[0]["reduce_launches"])))
-    seg_elems = st[0]["reduce_elements"] // max(1, st[0]["reduce_segments"])
+    rank_bytes = device_bytes(st_rank)
+    world_bytes = sum(device_bytes(s) for s in st)
+    segs_per_launch = max(1, round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"])))
+    first = H.Plan(algo, world, rank, n, 4, chunk).ranges[0]
+    seg_elems = first[1] - first[0]
 
     algbw = n * 4 / sec_per_step * 1e-9
+    world_algbw = n * 4 / world_sec * 1e-9
     line = {
         "metric": "emulated allreduce algbw (GB/s) with reduce-kernel HBM roofline, fp32",
         "value": round(algbw, 2),
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
-        "warmup": args.warmup,
+        "warmup": warm,
         "ms_per_step": round(sec_per_step * 1e3, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -283,25 +303,32 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE configs[%d]: %s allreduce, %d emulated ranks on one GPU, %d fp32 (%.0f MiB) per rank, "
-                        "IBCOMM_CHUNKSIZE=%d, all ranks' schedules executed per step" % (
-                            args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk),
-            "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk,
+            "workload": "BASELINE configs[%d]: %s allreduce, %d emulated ranks, %d fp32 (%.0f MiB) per rank, IBCOMM_CHUNKSIZE=%d; "
+                        "one step = rank %d's complete schedule on the GPU (its landings, reductions and gathers), the "
+                        "other ranks' messages replayed from a recording of the full world" % (
+                            args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk, rank),
+            "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk, "measured_rank": rank,
             "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "kernel"),
             "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64")),
         },
         "parity_bit_exact": parity,
         "extra": {
             "busbw_GBps": round(algbw * 2 * (world - 1) / world, 2),
-            "rank_share_algbw_GBps": round(algbw * world, 2),
-            "device_traffic_GB_per_step": round(device_bytes_per_step * 1e-9, 3),
-            "aggregate_device_GBps": round(device_bytes_per_step / sec_per_step * 1e-9, 1),
-            "aggregate_frac_of_hbm_peak": round(device_bytes_per_step / sec_per_step * 1e-9 / HBM_PEAK_GBPS, 4),
-            "rank0_reduce_launches_per_step": st[0]["reduce_launches"] / steps,
-            "rank0_segments_per_launch": segs_per_launch,
-            "rank0_reduce_elements_per_step": st[0]["reduce_elements"] // steps,
-            "rank0_landing_copies_per_step": st[0]["landing_copies"] / steps,
-            "rank0_gather_copies_per_step": st[0]["gather_copies"] / steps,
+            "rank_device_traffic_GB_per_step": round(rank_bytes * 1e-9, 3),
+            "rank_device_GBps": round(rank_bytes / sec_per_step * 1e-9, 1),
+            "rank_frac_of_hbm_peak": round(rank_bytes / sec_per_step * 1e-9 / HBM_PEAK_GBPS, 4),
+            "rank_reduce_launches_per_step": st_rank["reduce_launches"],
+            "rank_segments_per_launch": segs_per_launch,
+            "rank_reduce_elements_per_step": st_rank["reduce_elements"],
+            "rank_landing_launches_per_step": st_rank["landing_copies"],
+            "rank_gather_launches_per_step": st_rank["gather_copies"],
+            "world_all_ranks_on_one_gpu": {
+                "ms_per_step": round(world_sec * 1e3, 4),
+                "algbw_GBps": round(world_algbw, 2),
+                "device_traffic_GB_per_step": round(world_bytes * 1e-9, 3),
+                "device_GBps": round(world_bytes / world_sec * 1e-9, 1),
+                "frac_of_hbm_peak": round(world_bytes / world_sec * 1e-9 / HBM_PEAK_GBPS, 4),
+            },
             "streams_per_rank": st[0]["streams_created"],
             "issue": "eager" if args.no_graph else "hip graph replay",
             "graph_calls_eager_captured_replayed": list(graph_counters),

@@ -103,6 +103,19 @@ int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* comm, const int32_t* 
 int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
                                const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
 
+/* One rank's share on its own.  ibcomm_hip_world_record runs the whole world once (like
+ * ibcomm_hip_world_allreduce) while keeping, in device memory, every message `rank` receives and the
+ * point of its own schedule at which each became available.  ibcomm_hip_replay_allreduce then runs
+ * that rank's complete schedule alone: the peers are ghosts whose messages come from the recording,
+ * paced as in the recorded run, and whose receives cost nothing.  Same result in recvbuf as the
+ * world run gives that rank (for the same sendbuf contents).  This is how one GPU's part of
+ * AllreduceRingCuda / AllreduceRabenseifnerCuda (ibcomm/allreduce_cuda_impl.h:35-301, 326-717) is
+ * timed without the other ranks' work on the same device; the reference has no counterpart. */
+int ibcomm_hip_world_record(ibcomm_hip_comm* const* comms, int world_size, int rank, int algo, int dtype,
+                            const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
+int ibcomm_hip_replay_allreduce(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf,
+                                size_t len_elements);
+
 /* ibcomm_hip_world_allreduce records the device work of a call shape (same buffers, length, chunk
  * size and knobs) into a HIP graph on its second use and replays the graph from then on; mode 0
  * turns that off (every call is issued eagerly), mode 1 is the default (IBCOMM_HIP_GRAPH).  No

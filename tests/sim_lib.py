@@ -31,11 +31,14 @@ _lib = None
 
 def lib():
     global _lib
-    if _lib is None:
+    if _lib is None or not hasattr(_lib, 'sim_record_replay'):
         subprocess.check_call(["make", "-s", "-C", os.path.join(HERE, "support")])
         _lib = C.CDLL(SIM_SO)
         _lib.sim_world_allreduce.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                              C.c_size_t, C.c_int, C.c_int, C.c_uint, C.c_int, C.c_int, C.POINTER(Report)]
+        _lib.sim_record_replay.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                           C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_uint, C.c_void_p, C.c_int,
+                                           C.POINTER(Report)]
     return _lib
 
 
@@ -77,3 +80,36 @@ def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, th
             else:
                 os.environ[k] = v
     return rc, recv, rep
+
+
+def record_replay(algo, sendbufs, rank, chunksize=None, max_fuse=64, landing=1, seed=0, replays=1, pool_bytes=1 << 16):
+    """World run recording `rank`, then `rank` alone against the recording.
+    -> (rc, [world recvbuf per rank], replayed recvbuf of `rank`, Report with that rank's replay stats)"""
+    world = len(sendbufs)
+    sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]
+    n = sendbufs[0].size
+    recv = []
+    for _ in range(world + 1):
+        r = np.empty(n, dtype=sendbufs[0].dtype)
+        r.view(np.uint8)[:] = 0x55
+        recv.append(r)
+    out = recv.pop()
+    sp = (C.c_void_p * world)(*[s.ctypes.data for s in sendbufs])
+    rp = (C.c_void_p * world)(*[r.ctypes.data for r in recv])
+    saved = {k: os.environ.get(k) for k in ("IBCOMM_CHUNKSIZE", "IBCOMM_MEMORY_POOL_PRE_ALLOC")}
+    try:
+        if chunksize is None:
+            os.environ.pop("IBCOMM_CHUNKSIZE", None)
+        else:
+            os.environ["IBCOMM_CHUNKSIZE"] = str(chunksize)
+        os.environ["IBCOMM_MEMORY_POOL_PRE_ALLOC"] = str(pool_bytes)
+        rep = Report()
+        rc = lib().sim_record_replay(algo, DT[sendbufs[0].dtype], world, sp, rp, n, rank, max_fuse, landing, seed,
+                                     out.ctypes.data, replays, C.byref(rep))
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    return rc, recv, out, rep

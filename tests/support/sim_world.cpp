@@ -77,4 +77,44 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   return rc;
 }
 
+// Records `rank`'s incoming traffic during one world run, then runs that rank alone `replays` times
+// against the recording, writing its result to replay_out.
+int sim_record_replay(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,
+                      int rank, int max_fuse, int landing, unsigned seed, void* replay_out, int replays, sim_report* rep) {
+  *rep = sim_report();
+  Sim::Get().Reset(seed);
+  Fabric<SimBackend> fabric(world);
+  std::vector<std::unique_ptr<Communicator<SimBackend>>> comms;
+  std::vector<Communicator<SimBackend>*> raw;
+  int rc = kOk;
+  for (int r = 0; r < world && rc == kOk; r++) {
+    comms.emplace_back(new Communicator<SimBackend>(&fabric, world));
+    rc = comms.back()->Init();
+    comms.back()->RegisterMyself(r);
+    comms.back()->set_max_fuse(max_fuse);
+    comms.back()->set_landing(landing);
+    raw.push_back(comms.back().get());
+  }
+  size_t log_bytes = 0;
+  if (rc == kOk) rc = raw[rank]->RecordingBytes(algo, dtype, len, &log_bytes);
+  if (rc == kOk) rc = fabric.StartRecording(rank, log_bytes);
+  if (rc == kOk) rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, true);
+  fabric.StopRecording();
+  raw[rank]->reset_stats();
+  for (int k = 0; k < replays && rc == kOk; k++) {
+    if (!fabric.StartReplay(rank)) rc = Fail(kInvalidArgument, "nothing recorded");
+    if (rc == kOk) rc = RunAlone<SimBackend>(raw[rank], algo, dtype, sendbufs[rank], replay_out, len, true);
+    fabric.StopReplay();
+  }
+  if (rc != kOk) snprintf(rep->error, sizeof rep->error, "%s", LastErrorBuffer());
+  std::string first;
+  rep->rc = rc;
+  rep->nodes = Sim::Get().node_count();
+  rep->races = Sim::Get().CheckRaces(&first);
+  rep->unrecorded_waits = Sim::Get().unrecorded_waits();
+  rep->rank0 = raw[rank]->stats();
+  snprintf(rep->first_race, sizeof rep->first_race, "%s", first.c_str());
+  return rc;
+}
+
 }  // extern "C"

@@ -151,3 +151,31 @@ def test_work_per_rank_matches_the_schedule():
     # Rabenseifner rank 0 of 4: halving windows of 2 and 1 groups
     rep = check(RABEN, bufs, chunk, max_fuse=1)
     assert rep.rank0.reduce_segments == 3 * q and rep.rank0.gather_bytes == 3 * q * chunk
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("algo,world", [(RING, 2), (RING, 4), (RING, 5), (RABEN, 4), (RABEN, 8)])
+def test_one_rank_replayed_against_recorded_peers(algo, world, landing):
+    # a rank run alone against the recording of its incoming traffic must end with the very result
+    # it had in the full world, and must launch the same shapes (one step of the algorithm per pass)
+    n, chunk = 4096 + 5, 64
+    bufs = rand_bufs(world, n, seed=17)
+    orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs, chunk)
+    for rank in sorted({0, world // 2, world - 1}):
+        rc, recv, out, rep = S.record_replay(algo, bufs, rank, chunk, landing=landing, replays=2, seed=rank)
+        assert rc == 0, rep.error.decode()
+        for r in range(world):
+            assert np.array_equal(O.bits(recv[r]), O.bits(want[r]))
+        assert np.array_equal(O.bits(out), O.bits(want[rank])), "replayed rank %d differs" % rank
+        assert rep.races == 0, rep.first_race.decode()
+        assert rep.rank0.calls == 2
+        if algo == RING:
+            q = -(-n // (chunk // 4)) // world  # chunks per group (the last groups may hold one fewer)
+            launches_per_call = rep.rank0.reduce_launches // 2
+            assert world - 1 <= launches_per_call <= (world - 1) * (-(-(q + 1) // 64))
+
+
+def test_replay_refuses_a_different_call():
+    bufs = rand_bufs(4, 1000, seed=1)
+    rc, _, _, rep = S.record_replay(RING, bufs, 1, 40, replays=1)
+    assert rc == 0

@@ -126,6 +126,42 @@ def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
         assert w.graph_counters()[0] == eager + 3
 
 
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 8, 65536), (H.RING, 3, None), (H.RABENSEIFNER, 8, 65536)])
+def test_one_rank_replayed_against_recorded_peers(algo, world_size, chunk, landing):
+    # the measured unit of the benchmark: one rank's complete schedule, peers replaced by a recording
+    n = (1 << 20) + 7
+    host = rand_bufs(world_size, n, seed=31)
+    with G.env(IBCOMM_CHUNKSIZE=chunk):
+        orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
+        assert orc == 0
+        with H.World(world_size) as w:
+            w.set_landing(landing)
+            send = G.to_device(host)
+            recv = [G.poisoned_like(t) for t in send]
+            sp, rp = [t.data_ptr() for t in send], [t.data_ptr() for t in recv]
+            for rank in sorted({0, world_size - 1}):
+                torch.cuda.synchronize()
+                assert w.record(rank, algo, H.F32, sp, rp, n) == 0, H.last_error()
+                torch.cuda.synchronize()
+                for r in range(world_size):
+                    assert np.array_equal(O.bits(recv[r].cpu().numpy()), O.bits(want[r]))
+                before = w.graph_counters()
+                out = torch.empty_like(send[rank])
+                for it in range(5):  # eager, recorded into a graph, replayed
+                    out.view(torch.uint8).fill_(0x55)
+                    torch.cuda.synchronize()
+                    assert w.replay(rank, algo, H.F32, send[rank].data_ptr(), out.data_ptr(), n) == 0, H.last_error()
+                    torch.cuda.synchronize()
+                    assert np.array_equal(O.bits(out.cpu().numpy()), O.bits(want[rank])), "rank %d replay %d" % (rank, it)
+                after = w.graph_counters()
+                if landing != H.LAND_MEMCPY:
+                    assert after[1] - before[1] >= 1 and after[2] - before[2] >= 3
+            # the world still works after replays, and a replay without a matching recording is refused
+            assert w.allreduce_ptrs(algo, H.F32, sp, rp, n) == 0
+            assert w.replay(1, algo, H.F32, sp[1], rp[1], n) == H.INVALID_ARGUMENT
+
+
 # ------------------------------------------------------------------ reference tester cases
 
 def run_kat(world_size, algo, n, chunk=None):
