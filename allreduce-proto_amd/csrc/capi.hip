@@ -114,6 +114,7 @@ int ibcomm_hip_comm_create(ibcomm_hip_fabric* fabric, int world_size, ibcomm_hip
 int ibcomm_hip_comm_destroy(ibcomm_hip_comm* comm) {
   if (!comm) return kOk;
   comm->comm.Abort();
+  if (comm->comm.trace().enabled()) comm->comm.DumpTrace();  // the reference dumps in its destructor (cpp:145-147)
   comm->owner->DropGraphs();  // recorded graphs point into this communicator's pool
   comm->owner->has_last_eager = false;
   comm->owner->live_comms--;
@@ -457,6 +458,24 @@ int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode) {
   if (!comm) return Fail(kInvalidArgument, "comm is null");
   if (mode < kLandMemcpy || mode > kLandDirect) return Fail(kInvalidArgument, "landing mode must be 0, 1 or 2");
   comm->comm.set_landing(mode);
+  return kOk;
+}
+
+int ibcomm_hip_comm_set_timer_base(ibcomm_hip_comm* comm) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  comm->comm.trace().SetTimerBase();
+  return kOk;
+}
+
+int ibcomm_hip_comm_set_trace(ibcomm_hip_comm* comm, int enabled) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  comm->comm.trace().Enable(enabled != 0);
+  return kOk;
+}
+
+int ibcomm_hip_comm_dump_trace(ibcomm_hip_comm* comm) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  if (!comm->comm.DumpTrace()) return Fail(kInvalidArgument, "cannot write the trace file");
   return kOk;
 }
 

@@ -44,6 +44,7 @@
 #include "plan.hpp"
 #include "segments.hpp"
 #include "status.hpp"
+#include "trace.hpp"
 
 namespace ibcomm_hip {
 
@@ -109,7 +110,16 @@ class Communicator {
     // so no such buffer is allocated; the variable is still accepted so job scripts keep working.
     v = getenv("IBCOMM_WORK_GPU_MEMORY_SIZE");
     work_gpu_memory_size_ = v ? atoll(v) : (32ll << 20);
+    v = getenv("IBCOMM_HIP_TRACE");
+    trace_.Enable(v && atoi(v) != 0);
     return kOk;
+  }
+
+  Trace& trace() { return trace_; }
+  // DumpTrace (ibverbs_communicator.cpp:183-212): ${IBCOMM_TRACE_FILE:-ibcomm_trace}_<rank>.dat
+  bool DumpTrace() const {
+    const char* base = getenv("IBCOMM_TRACE_FILE");
+    return trace_.Dump(std::string(base ? base : "ibcomm_trace") + "_" + std::to_string(rank_) + ".dat");
   }
 
   void RegisterMyself(int rank) { rank_ = rank; }  // ibverbs_communicator.cpp:355-357
@@ -135,6 +145,7 @@ class Communicator {
   // ---- one collective: Begin, Progress until finished, Finish ------------------------------------
 
   int Begin(int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len_elements) {
+    TraceScope scope(&trace_, Trace::kOther);
     if (active_) return Fail(kNotSupported, "an allreduce is already in progress on this communicator");
     if (rank_ < 0 || rank_ >= world_size_) return Fail(kInvalidArgument, "RegisterMyself has not been called");
     es_ = DTypeSize(dtype);
@@ -218,6 +229,7 @@ class Communicator {
   // this returns, as in the reference (allreduce_cuda_impl.h:280-299, :709-715).
   int Finish(bool wait_pulls) {
     if (!active_) return kOk;
+    TraceScope scope(&trace_, Trace::kOther);
     int rc = pool_.SynchronizeStreams();
     if (rc == kOk && wait_pulls) {
       for (Event e : pull_events_) {
@@ -388,6 +400,7 @@ class Communicator {
         ready_stream = d.stream;
         has_ready = d.has_event;
       }
+      TraceScope scope(&trace_, Trace::kIssueSend);
       const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready, ready_stream);
       posted_[s.peer].push_back(PostedSend{ticket, static_cast<int>(next_send_)});
       if (s.dep >= 0 || in_place_) chunk_unconsumed_[s.chunk]++;
@@ -405,7 +418,11 @@ class Communicator {
       // A gather overwrites recvbuf[chunk]; a send of ours out of that range must have been read first.
       if (r.kind == kGather && chunk_unconsumed_[r.chunk] > 0) break;
       PendingRecv p;
-      if (!fabric_->Take(rank_, r.peer, &p.msg, next_send_)) break;
+      trace_.Mark(Trace::kReceived);
+      const bool got = fabric_->Take(rank_, r.peer, &p.msg, next_send_);
+      if (!got) trace_.Unmark(Trace::kReceived);
+      if (!got) break;
+      trace_.Mark(Trace::kReceived);
       if (p.msg.bytes != ChunkBytes(r.chunk))
         return Fail(kTransportError, "rank %d: message of %zu bytes from rank %d where chunk %d has %zu", rank_, p.msg.bytes,
                     r.peer, r.chunk, ChunkBytes(r.chunk));
@@ -421,7 +438,10 @@ class Communicator {
         // Segments of one launch run concurrently: a chunk whose previous partial sum is still
         // waiting in this batch must go into the next launch.
         if (chunk_in_batch_[r.chunk]) IBCOMM_RETURN_IF_ERROR(FlushReduces());
-        if (landing_ != kLandDirect) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+        if (landing_ != kLandDirect) {
+          TraceScope scope(&trace_, Trace::kIssueRecv);
+          IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+        }
         chunk_in_batch_[r.chunk] = 1;
         pending_reduce_.push_back(p);
         if (static_cast<int>(pending_reduce_.size()) >= max_fuse_) IBCOMM_RETURN_IF_ERROR(FlushReduces());
@@ -436,6 +456,7 @@ class Communicator {
   // Finished chunks: recvbuf[c] <- message.
   int FlushGathers() {
     if (pending_gather_.empty()) return kOk;
+    TraceScope scope(&trace_, Trace::kIssueCopyKernel);
     if (landing_ != kLandMemcpy) {
       Stream s;
       IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
@@ -491,6 +512,7 @@ class Communicator {
     Stream s{};
     std::vector<OpState> landed(n);
 
+    trace_.Mark(Trace::kIssueCopyKernel);
     if (landing_ == kLandMemcpy) {
       for (size_t i = 0; i < n; i++) {
         PendingRecv& p = pending_reduce_[i];
@@ -535,6 +557,8 @@ class Communicator {
       }
     }
 
+    trace_.Mark(Trace::kIssueCopyKernel);
+    trace_.Mark(Trace::kIssueReduKernel);
     SegmentBatch batch;
     batch.count = 0;
     for (size_t i = 0; i < n; i++) {
@@ -557,6 +581,8 @@ class Communicator {
     stats_.reduce_segments += n;
     OpState done;
     IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+    trace_.Mark(Trace::kIssueReduKernel);
+    TraceScope reduced(&trace_, Trace::kReduced);
     for (size_t i = 0; i < n; i++) {
       const PendingRecv& p = pending_reduce_[i];
       const RecvOp& r = plan_.recvs[p.op];
@@ -613,6 +639,7 @@ class Communicator {
   int arena_ = 0;
   size_t event_cursor_ = 0;
   EngineStats stats_;
+  Trace trace_;
 };
 
 }  // namespace ibcomm_hip

@@ -1,0 +1,92 @@
+// Host-side pipeline trace, in the reference's categories and file format.
+//
+// The reference compiles this in with -DUSE_TRACE: TRACE(v) pushes a CLOCK_MONOTONIC_RAW timestamp
+// (ibcomm/allreduce_cuda_impl.h:18-22, ibcomm/util.h:62-70), events come in begin/end pairs in seven
+// vectors (ibcomm/ibverbs_communicator.h:168-189), and the destructor writes
+// ${IBCOMM_TRACE_FILE:-ibcomm_trace}_<rank>.dat with one CSV line per category,
+// "name,start_ms,duration_ms,start_ms,duration_ms,..." in scientific notation relative to the timer
+// base (ibcomm/ibverbs_communicator.cpp:157-216).  Here tracing is switched on at run time
+// (IBCOMM_HIP_TRACE=1) and costs one branch per event when off.  What the categories mean for the
+// stream-ordered engine:
+//   received            a message was taken from a peer's channel
+//   reduced             the reduction of a batch of chunks was enqueued and its result handed on
+//   issue-send          a send was posted
+//   issue-copy-kernel   a landing copy or a gather was enqueued
+//   issue-redu-kernel   a reduction launch was enqueued
+//   issue-recv          a pool slot was reserved for an incoming message
+//   other               Begin / Finish of a collective
+#pragma once
+
+#include <time.h>
+
+#include <fstream>
+#include <string>
+#include <vector>
+
+namespace ibcomm_hip {
+
+class Trace {
+ public:
+  enum Category { kReceived, kReduced, kIssueSend, kIssueCopyKernel, kIssueReduKernel, kIssueRecv, kOther, kCategories };
+
+  void Enable(bool on) { enabled_ = on; }
+  bool enabled() const { return enabled_; }
+  void SetTimerBase() { clock_gettime(CLOCK_MONOTONIC_RAW, &base_); has_base_ = true; }  // cpp:214-216
+
+  void Mark(Category c) {
+    if (!enabled_) return;
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC_RAW, &ts);
+    if (!has_base_) { base_ = ts; has_base_ = true; }  // the reference leaves the base uninitialised unless SetTimerBase is called
+    events_[c].push_back(ts);
+  }
+
+  // Takes back the last Mark of a pair that turned out not to happen (a poll that found nothing).
+  void Unmark(Category c) {
+    if (enabled_ && !events_[c].empty()) events_[c].pop_back();
+  }
+
+  size_t pairs(Category c) const { return events_[c].size() / 2; }
+
+  // DumpTrace, cpp:183-212.
+  bool Dump(const std::string& path) const {
+    static const char* names[kCategories] = {"received", "reduced", "issue-send", "issue-copy-kernel",
+                                             "issue-redu-kernel", "issue-recv", "other"};
+    std::ofstream out(path.c_str());
+    if (!out.good()) return false;
+    out << std::scientific;
+    for (int c = 0; c < kCategories; c++) {
+      out << names[c] << ",";
+      const std::vector<struct timespec>& v = events_[c];
+      for (size_t i = 0; i + 1 < v.size(); i += 2) out << Millis(base_, v[i]) << "," << Millis(v[i], v[i + 1]) << ",";
+      out << std::endl;
+    }
+    return true;
+  }
+
+  void Clear() {
+    for (auto& v : events_) v.clear();
+  }
+
+ private:
+  static double Millis(const struct timespec& a, const struct timespec& b) {
+    return (b.tv_sec - a.tv_sec) * 1e3 + (b.tv_nsec - a.tv_nsec) * 1e-6;
+  }
+  bool enabled_ = false;
+  bool has_base_ = false;
+  struct timespec base_ = {};
+  std::vector<struct timespec> events_[kCategories];
+};
+
+// Begin/end pair around a scope.
+class TraceScope {
+ public:
+  TraceScope(Trace* t, Trace::Category c) : t_(t), c_(c) { t_->Mark(c_); }
+  ~TraceScope() { t_->Mark(c_); }
+
+ private:
+  Trace* t_;
+  Trace::Category c_;
+};
+
+}  // namespace ibcomm_hip

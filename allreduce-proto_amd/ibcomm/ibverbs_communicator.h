@@ -96,6 +96,10 @@ class IBVerbsCommunicator {
                       "AllreduceRabenseifner on host buffers is not part of the HIP build; use AllreduceRabenseifnerCuda.");
   }
 
+  // ibverbs_communicator.cpp:157-216; the trace is recorded when IBCOMM_HIP_TRACE=1.
+  void SetTimerBase() { ibcomm_hip_comm_set_timer_base(comm_); }
+  void DumpTrace() const { ibcomm_hip_comm_dump_trace(comm_); }
+
   ibcomm_hip_comm* handle() { return comm_; }
 
  private:

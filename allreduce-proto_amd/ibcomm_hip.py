@@ -27,6 +27,7 @@ EXPORTS = [
     "ibcomm_hip_rank_to_chunk", "ibcomm_hip_get_exp_of_two", "ibcomm_hip_plan_create", "ibcomm_hip_plan_destroy",
     "ibcomm_hip_plan_counts", "ibcomm_hip_plan_range", "ibcomm_hip_plan_recv", "ibcomm_hip_plan_send",
     "ibcomm_hip_fabric_set_graph_mode", "ibcomm_hip_fabric_graph_counters", "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
+    "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
 ]
 
 
@@ -82,6 +83,9 @@ def lib():
     L.ibcomm_hip_comm_set_landing.argtypes = [vp, i]
     L.ibcomm_hip_comm_stats.argtypes = [vp, C.POINTER(Stats)]
     L.ibcomm_hip_comm_reset_stats.argtypes = [vp]
+    L.ibcomm_hip_comm_set_trace.argtypes = [vp, i]
+    L.ibcomm_hip_comm_set_timer_base.argtypes = [vp]
+    L.ibcomm_hip_comm_dump_trace.argtypes = [vp]
     _lib = L
     return L
 
@@ -213,6 +217,16 @@ class World:
         for t in th:
             t.join()
         return rcs, msgs
+
+    def set_trace(self, enabled=True):
+        for h in self.comms:
+            lib().ibcomm_hip_comm_set_trace(h, 1 if enabled else 0)
+            lib().ibcomm_hip_comm_set_timer_base(h)
+
+    def dump_trace(self):
+        """Writes ${IBCOMM_TRACE_FILE:-ibcomm_trace}_<rank>.dat for every rank."""
+        for h in self.comms:
+            assert lib().ibcomm_hip_comm_dump_trace(h) == 0, last_error()
 
     def stats(self, rank=0):
         s = Stats()

@@ -166,6 +166,16 @@ int ibcomm_hip_comm_set_max_fuse(ibcomm_hip_comm* comm, int max_chunks_per_launc
  * launch for all messages of a pass, 2 = the reduction reads the sender's buffer directly. */
 int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode);
 
+/* Host-side pipeline trace in the reference's seven categories and .dat format
+ * (IBVerbsCommunicator::SetTimerBase / DumpTrace, ibcomm/ibverbs_communicator.cpp:157-216; TRACE()
+ * call sites in ibcomm/allreduce_cuda_impl.h).  The reference compiles it in with -DUSE_TRACE and
+ * dumps in the destructor; here it is switched on with IBCOMM_HIP_TRACE=1 or set_trace, dumped by
+ * dump_trace and by comm_destroy, to ${IBCOMM_TRACE_FILE:-ibcomm_trace}_<rank>.dat.  Graph replays
+ * do no host-side pipeline work and therefore add no events. */
+int ibcomm_hip_comm_set_trace(ibcomm_hip_comm* comm, int enabled);
+int ibcomm_hip_comm_set_timer_base(ibcomm_hip_comm* comm);
+int ibcomm_hip_comm_dump_trace(ibcomm_hip_comm* comm);
+
 typedef struct {
   uint64_t calls;
   uint64_t reduce_launches;

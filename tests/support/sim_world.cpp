@@ -77,6 +77,51 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   return rc;
 }
 
+// Runs one world allreduce with tracing on and dumps rank 0's trace to `path`.
+int sim_trace(int algo, int world, const void* const* sendbufs, void* const* recvbufs, size_t len, int max_fuse,
+              const char* path, unsigned long long* pairs /* 7 */) {
+  Sim::Get().Reset(3);
+  Fabric<SimBackend> fabric(world);
+  std::vector<std::unique_ptr<Communicator<SimBackend>>> comms;
+  std::vector<Communicator<SimBackend>*> raw;
+  for (int r = 0; r < world; r++) {
+    comms.emplace_back(new Communicator<SimBackend>(&fabric, world));
+    if (comms.back()->Init() != kOk) return 1;
+    comms.back()->RegisterMyself(r);
+    comms.back()->set_max_fuse(max_fuse);
+    comms.back()->trace().Enable(true);
+    comms.back()->trace().SetTimerBase();
+    raw.push_back(comms.back().get());
+  }
+  const int rc = RunWorld<SimBackend>(raw.data(), world, algo, kF32, sendbufs, recvbufs, len, true);
+  if (rc != kOk) return rc;
+  for (int c = 0; c < Trace::kCategories; c++) pairs[c] = raw[0]->trace().pairs(static_cast<Trace::Category>(c));
+  return raw[0]->trace().Dump(path) ? kOk : 1;
+}
+
+// Pool knobs and controller rules (memory_pool.h:111-121, 139-173): returns the status of creating a
+// communicator under the current environment, and in *second_controller the status of asking the
+// pool for a second controller while one is live.
+int sim_pool_rules(int* second_controller, unsigned long long* block_bytes, int* max_streams, int* slots_for_chunk,
+                   unsigned long long chunk_bytes) {
+  Sim::Get().Reset(1);
+  Fabric<SimBackend> fabric(2);
+  Communicator<SimBackend> c(&fabric, 2);
+  const int rc = c.Init();
+  if (rc != kOk) return rc;
+  *block_bytes = c.pool().block_bytes();
+  *max_streams = c.pool().max_streams();
+  MemoryController<SimBackend> a, b;
+  int rc2 = c.pool().GetController(chunk_bytes, &a);
+  if (rc2 != kOk) return rc2;
+  *slots_for_chunk = static_cast<int>(a.slot_count());
+  *second_controller = c.pool().GetController(chunk_bytes, &b);
+  a.Release();
+  rc2 = c.pool().GetController(chunk_bytes, &b);  // free again after release
+  b.Release();
+  return rc2;
+}
+
 // Records `rank`'s incoming traffic during one world run, then runs that rank alone `replays` times
 // against the recording, writing its result to replay_out.
 int sim_record_replay(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,

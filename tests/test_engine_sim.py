@@ -179,3 +179,89 @@ def test_replay_refuses_a_different_call():
     bufs = rand_bufs(4, 1000, seed=1)
     rc, _, _, rep = S.record_replay(RING, bufs, 1, 40, replays=1)
     assert rc == 0
+
+
+def pool_rules(chunk_bytes=4096, **env):
+    import ctypes as C
+    import os
+    L = S.lib()
+    L.sim_pool_rules.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_ulonglong), C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                 C.c_ulonglong]
+    keys = ("IBCOMM_NUM_CUDA_STREAM", "IBCOMM_MEMORY_POOL_PRE_ALLOC", "IBCOMM_HIP_MAX_FUSE", "IBCOMM_HIP_LANDING")
+    saved = {k: os.environ.get(k) for k in keys}
+    try:
+        for k in keys:
+            os.environ.pop(k, None)
+        os.environ["IBCOMM_MEMORY_POOL_PRE_ALLOC"] = "65536"
+        for k, v in env.items():
+            os.environ[k] = str(v)
+        second, block, streams, slots = C.c_int(-1), C.c_ulonglong(0), C.c_int(0), C.c_int(0)
+        rc = L.sim_pool_rules(C.byref(second), C.byref(block), C.byref(streams), C.byref(slots), chunk_bytes)
+        return rc, second.value, block.value, streams.value, slots.value
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+def test_pool_knobs_and_single_controller_rule():
+    # defaults and the one-controller-at-a-time rule (memory_pool.h:111-121 -> NOT_SUPPORTED)
+    rc, second, block, streams, slots = pool_rules()
+    assert rc == 0 and second == 4 and block == 65536 and streams == 8
+    # every slot that fits is used: stride = round_up(4096 + 16, 256) = 4352 -> 15 slots in 64 KiB
+    assert slots == 65536 // 4352 == 15
+    # IBCOMM_NUM_CUDA_STREAM must be in (0, 1024] (memory_pool.h:139-154 -> INVALID_ARGUMENT)
+    for bad in ("0", "-1", "1025", "abc"):
+        assert pool_rules(IBCOMM_NUM_CUDA_STREAM=bad)[0] == 1
+    assert pool_rules(IBCOMM_NUM_CUDA_STREAM="1024")[3] == 1024
+    assert pool_rules(IBCOMM_NUM_CUDA_STREAM="64")[3] == 64
+    # IBCOMM_MEMORY_POOL_PRE_ALLOC below 4 is refused (memory_pool.h:158-173); the 1 GiB ceiling is lifted
+    for bad in ("3", "0", "-5", "x"):
+        assert pool_rules(IBCOMM_MEMORY_POOL_PRE_ALLOC=bad)[0] == 1
+    assert pool_rules(IBCOMM_MEMORY_POOL_PRE_ALLOC="131072")[2] == 131072
+    # this build's own knobs are validated too
+    assert pool_rules(IBCOMM_HIP_MAX_FUSE="0")[0] == 1
+    assert pool_rules(IBCOMM_HIP_MAX_FUSE="65")[0] == 1
+    assert pool_rules(IBCOMM_HIP_LANDING="bogus")[0] == 1
+    assert pool_rules(IBCOMM_HIP_LANDING="direct")[0] == 0
+
+
+def test_trace_file_has_the_reference_format(tmp_path):
+    # ibcomm/ibverbs_communicator.cpp:157-212: seven lines "name,start_ms,dur_ms,...", scientific notation
+    import ctypes as C
+    import os
+    world, n = 4, 4096
+    bufs = rand_bufs(world, n, seed=2)
+    recv = [np.empty_like(b) for b in bufs]
+    L = S.lib()
+    L.sim_trace.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_size_t, C.c_int, C.c_char_p,
+                            C.POINTER(C.c_ulonglong)]
+    pairs = (C.c_ulonglong * 7)()
+    path = str(tmp_path / "trace_0.dat")
+    os.environ["IBCOMM_CHUNKSIZE"] = "1024"
+    os.environ["IBCOMM_MEMORY_POOL_PRE_ALLOC"] = "65536"
+    try:
+        rc = L.sim_trace(RING, world, (C.c_void_p * world)(*[b.ctypes.data for b in bufs]),
+                         (C.c_void_p * world)(*[r.ctypes.data for r in recv]), n, 1, path.encode(), pairs)
+    finally:
+        os.environ.pop("IBCOMM_CHUNKSIZE")
+        os.environ.pop("IBCOMM_MEMORY_POOL_PRE_ALLOC")
+    assert rc == 0
+    lines = open(path).read().splitlines()
+    names = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
+    assert [ln.split(",")[0] for ln in lines] == names
+    q = n * 4 // 1024 // world  # chunks per group
+    want_pairs = {"received": 2 * (world - 1) * q, "reduced": (world - 1) * q, "issue-send": 2 * (world - 1) * q,
+                  "issue-redu-kernel": (world - 1) * q, "issue-recv": (world - 1) * q, "other": 2}
+    for k, ln in enumerate(lines):
+        fields = ln.split(",")
+        assert fields[-1] == ""  # every value is followed by a comma
+        vals = [float(x) for x in fields[1:-1]]
+        assert len(vals) == 2 * pairs[k]
+        assert all("e" in x for x in fields[1:-1])  # std::scientific
+        starts, durs = vals[0::2], vals[1::2]
+        assert all(d >= 0 for d in durs) and starts == sorted(starts) and all(s >= 0 for s in starts)
+        if names[k] in want_pairs:
+            assert pairs[k] == want_pairs[names[k]], names[k]
