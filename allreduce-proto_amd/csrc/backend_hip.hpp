@@ -67,6 +67,11 @@ struct HipBackend {
     IBCOMM_HIP_CHECK(hipEventSynchronize(e));
     return kOk;
   }
+  // Blocking copy between any two buffers, host or device (point-to-point Send/Recv).
+  static int CopySync(void* dst, const void* src, size_t bytes) {
+    IBCOMM_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDefault));
+    return kOk;
+  }
   static int CopyAsync(void* dst, const void* src, size_t bytes, Stream s) {
     IBCOMM_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
     return kOk;

@@ -461,6 +461,41 @@ int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode) {
   return kOk;
 }
 
+int ibcomm_hip_send(ibcomm_hip_comm* comm, int dest_rank, const void* buf, size_t len, int blocking) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  return comm->comm.Send(dest_rank, buf, len, blocking != 0);
+}
+int ibcomm_hip_recv(ibcomm_hip_comm* comm, int src_rank, void* buf, size_t len, int blocking) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  return comm->comm.Recv(src_rank, buf, len, blocking != 0);
+}
+int ibcomm_hip_send_poll(ibcomm_hip_comm* comm, int dest_rank, int* completed) {
+  if (!comm || !completed) return Fail(kInvalidArgument, "null argument");
+  bool ok = false;
+  const int rc = comm->comm.SendPoll(dest_rank, &ok);
+  *completed = ok ? 1 : 0;
+  return rc;
+}
+int ibcomm_hip_recv_poll(ibcomm_hip_comm* comm, int src_rank, int* completed) {
+  if (!comm || !completed) return Fail(kInvalidArgument, "null argument");
+  bool ok = false;
+  const int rc = comm->comm.RecvPoll(src_rank, &ok);
+  *completed = ok ? 1 : 0;
+  return rc;
+}
+int ibcomm_hip_send_wait(ibcomm_hip_comm* comm, int dest_rank) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  return comm->comm.SendWait(dest_rank);
+}
+int ibcomm_hip_recv_wait(ibcomm_hip_comm* comm, int src_rank) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  return comm->comm.RecvWait(src_rank);
+}
+int ibcomm_hip_bcast(ibcomm_hip_comm* comm, void* buf, size_t len, int root) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  return comm->comm.Bcast(buf, len, root);
+}
+
 int ibcomm_hip_comm_set_timer_base(ibcomm_hip_comm* comm) {
   if (!comm) return Fail(kInvalidArgument, "comm is null");
   comm->comm.trace().SetTimerBase();

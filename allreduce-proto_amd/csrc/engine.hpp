@@ -293,6 +293,63 @@ class Communicator {
     return kOk;
   }
 
+  // ---- point-to-point messaging over the loopback -------------------------------------------------
+  // IBVerbsCommunicator::Send / Recv / SendPoll / RecvPoll / SendWait / RecvWait / Bcast
+  // (ibcomm/ibverbs_communicator.cpp:371-384, 486-499, 416-473, 529-606).  Buffers may be host or
+  // device memory.  As in the reference, one non-blocking send and one non-blocking receive per peer
+  // may be outstanding; posting another before its Wait is NOT_SUPPORTED (cpp:375-378, 490-493).
+  // The receiver moves the data when it polls.
+
+  int Send(int dest, const void* buf, size_t len, bool blocking) {
+    IBCOMM_RETURN_IF_ERROR(CheckPeer(dest));
+    if (p2p_send_pending_[dest]) return Fail(kNotSupported, "SendWait must be called before next non-blocking send.");
+    fabric_->PostSend(rank_, dest, buf, len, Event{}, false);
+    p2p_send_pending_[dest] = 1;
+    return blocking ? SendWait(dest) : kOk;
+  }
+  int Recv(int src, void* buf, size_t len, bool blocking) {
+    IBCOMM_RETURN_IF_ERROR(CheckPeer(src));
+    if (p2p_recv_[src].active) return Fail(kNotSupported, "RecvWait must be called before next non-blocking send.");
+    p2p_recv_[src].buf = buf;
+    p2p_recv_[src].len = len;
+    p2p_recv_[src].active = true;
+    return blocking ? RecvWait(src) : kOk;
+  }
+  int SendPoll(int dest, bool* completed) {
+    IBCOMM_RETURN_IF_ERROR(CheckPeer(dest));
+    typename Fabric<B>::Completion c;
+    *completed = fabric_->PollSendCompletion(rank_, dest, &c);
+    if (*completed) p2p_send_pending_[dest] = 0;
+    return kOk;
+  }
+  int RecvPoll(int src, bool* completed) {
+    IBCOMM_RETURN_IF_ERROR(CheckPeer(src));
+    *completed = false;
+    if (!p2p_recv_[src].active) return kOk;
+    Message m;
+    if (!fabric_->Take(rank_, src, &m)) return kOk;
+    if (m.bytes > p2p_recv_[src].len)
+      return Fail(kTransportError, "message of %zu bytes from rank %d does not fit the posted buffer of %zu", m.bytes, src,
+                  p2p_recv_[src].len);
+    const int rc = B::CopySync(p2p_recv_[src].buf, m.src, m.bytes);
+    fabric_->Complete(rank_, src, m.ticket, Event{}, false);
+    p2p_recv_[src].active = false;
+    *completed = true;
+    return rc;
+  }
+  int SendWait(int dest) { return SpinUntil([&](bool* ok) { return SendPoll(dest, ok); }, "SendWait", dest); }
+  int RecvWait(int src) { return SpinUntil([&](bool* ok) { return RecvPoll(src, ok); }, "RecvWait", src); }
+  // Naive broadcast (cpp:586-606): the root sends to everyone, then waits for every send.
+  int Bcast(void* buf, size_t len, int root) {
+    IBCOMM_RETURN_IF_ERROR(CheckPeer(root));
+    if (rank_ != root) return Recv(root, buf, len, true);
+    for (int i = 0; i < world_size_; i++)
+      if (i != rank_) IBCOMM_RETURN_IF_ERROR(Send(i, buf, len, false));
+    for (int i = 0; i < world_size_; i++)
+      if (i != rank_) IBCOMM_RETURN_IF_ERROR(SendWait(i));
+    return kOk;
+  }
+
   const Plan& plan() const { return plan_; }
   bool active() const { return active_; }
   size_t recv_cursor() const { return next_recv_; }
@@ -315,6 +372,11 @@ class Communicator {
   struct PostedSend {
     uint64_t ticket;
     int send_index;
+  };
+  struct PostedRecv {
+    void* buf = nullptr;
+    size_t len = 0;
+    bool active = false;
   };
 
   char* RecvPtr(int chunk) const { return recvbuf_ + plan_.part.ranges[chunk].begin * es_; }
@@ -602,6 +664,32 @@ class Communicator {
     return B::CopyAsync(m.record_to, m.src, m.bytes, s);
   }
 
+  int CheckPeer(int peer) {
+    if (rank_ < 0) return Fail(kInvalidArgument, "RegisterMyself has not been called");
+    if (peer < 0 || peer >= world_size_) return Fail(kInvalidArgument, "rank %d outside world of %d", peer, world_size_);
+    if (active_) return Fail(kNotSupported, "point-to-point calls cannot be mixed into a running allreduce");
+    if (p2p_send_pending_.empty()) {
+      p2p_send_pending_.assign(world_size_, 0);
+      p2p_recv_.assign(world_size_, PostedRecv());
+    }
+    return kOk;
+  }
+
+  template <class Poll>
+  int SpinUntil(Poll poll, const char* what, int peer) {
+    const char* t = getenv("IBCOMM_HIP_TIMEOUT_S");
+    const double limit = t ? atof(t) : 120.0;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+      bool ok = false;
+      IBCOMM_RETURN_IF_ERROR(poll(&ok));
+      if (ok) return kOk;
+      std::this_thread::yield();
+      if (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > limit)
+        return Fail(kTransportError, "rank %d: %s(%d) saw no completion for %.0f s", rank_, what, peer, limit);
+    }
+  }
+
   int WaitOnSlot(Stream s, const Memory<B>* slot) {
     if (!slot->has_free_event || slot->free_stream == s) return kOk;
     stats_.stream_waits++;
@@ -640,6 +728,8 @@ class Communicator {
   size_t event_cursor_ = 0;
   EngineStats stats_;
   Trace trace_;
+  std::vector<char> p2p_send_pending_;   // per peer: a non-blocking Send awaits its SendPoll/SendWait
+  std::vector<PostedRecv> p2p_recv_;     // per peer: the buffer a non-blocking Recv posted
 };
 
 }  // namespace ibcomm_hip

@@ -73,6 +73,27 @@ class IBVerbsCommunicator {
     Check(ibcomm_hip_comm_register_myself(comm_, my_rank), __LINE__);
   }
 
+  // Point-to-point messaging over the loopback (ibverbs_communicator.cpp:371-606); host or device buffers.
+  void Send(int dest_rank, const void* buf, size_t len, bool blocking = true) {
+    Check(ibcomm_hip_send(comm_, dest_rank, buf, len, blocking ? 1 : 0), __LINE__);
+  }
+  void Recv(int src_rank, void* buf, size_t len, bool blocking = true) {
+    Check(ibcomm_hip_recv(comm_, src_rank, buf, len, blocking ? 1 : 0), __LINE__);
+  }
+  bool SendPoll(int dest_rank) {
+    int done = 0;
+    Check(ibcomm_hip_send_poll(comm_, dest_rank, &done), __LINE__);
+    return done != 0;
+  }
+  bool RecvPoll(int src_rank) {
+    int done = 0;
+    Check(ibcomm_hip_recv_poll(comm_, src_rank, &done), __LINE__);
+    return done != 0;
+  }
+  void SendWait(int dest_rank) { Check(ibcomm_hip_send_wait(comm_, dest_rank), __LINE__); }
+  void RecvWait(int src_rank) { Check(ibcomm_hip_recv_wait(comm_, src_rank), __LINE__); }
+  void Bcast(void* buf, size_t len, int root) { Check(ibcomm_hip_bcast(comm_, buf, len, root), __LINE__); }
+
   // Device buffers.  Blocking; every rank of the world must be inside the same call.
   template <typename T>
   void AllreduceRingCuda(const T* sendbuf, T* recvbuf, size_t len_elements) {

@@ -27,7 +27,8 @@ EXPORTS = [
     "ibcomm_hip_rank_to_chunk", "ibcomm_hip_get_exp_of_two", "ibcomm_hip_plan_create", "ibcomm_hip_plan_destroy",
     "ibcomm_hip_plan_counts", "ibcomm_hip_plan_range", "ibcomm_hip_plan_recv", "ibcomm_hip_plan_send",
     "ibcomm_hip_fabric_set_graph_mode", "ibcomm_hip_fabric_graph_counters", "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
-    "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
+    "ibcomm_hip_send", "ibcomm_hip_recv", "ibcomm_hip_send_poll", "ibcomm_hip_recv_poll", "ibcomm_hip_send_wait",
+    "ibcomm_hip_recv_wait", "ibcomm_hip_bcast", "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
 ]
 
 
@@ -83,6 +84,13 @@ def lib():
     L.ibcomm_hip_comm_set_landing.argtypes = [vp, i]
     L.ibcomm_hip_comm_stats.argtypes = [vp, C.POINTER(Stats)]
     L.ibcomm_hip_comm_reset_stats.argtypes = [vp]
+    L.ibcomm_hip_send.argtypes = [vp, i, vp, sz, i]
+    L.ibcomm_hip_recv.argtypes = [vp, i, vp, sz, i]
+    L.ibcomm_hip_send_poll.argtypes = [vp, i, C.POINTER(i)]
+    L.ibcomm_hip_recv_poll.argtypes = [vp, i, C.POINTER(i)]
+    L.ibcomm_hip_send_wait.argtypes = [vp, i]
+    L.ibcomm_hip_recv_wait.argtypes = [vp, i]
+    L.ibcomm_hip_bcast.argtypes = [vp, vp, sz, i]
     L.ibcomm_hip_comm_set_trace.argtypes = [vp, i]
     L.ibcomm_hip_comm_set_timer_base.argtypes = [vp]
     L.ibcomm_hip_comm_dump_trace.argtypes = [vp]

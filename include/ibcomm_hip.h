@@ -134,6 +134,22 @@ int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, cons
                                const void* const* b, const size_t* len_elements, void* stream);
 int ibcomm_hip_max_segments(void);
 
+/* ---- point-to-point messaging over the loopback ------------------------------------------------ */
+
+/* IBVerbsCommunicator::Send / Recv (ibcomm/ibverbs_communicator.cpp:371-384, 486-499), SendPoll /
+ * RecvPoll (:416-461, 529-572), SendWait / RecvWait (:463-473, 574-584) and Bcast (:586-606).
+ * Buffers may be host or device memory; len is in bytes.  One non-blocking send and one non-blocking
+ * receive per peer may be outstanding: posting another before the matching Wait returns 4 with the
+ * reference's message.  *completed is 1 once per finished operation, else 0; polls never block.
+ * The receiving side moves the data when it polls or waits.  Each rank calls from its own thread. */
+int ibcomm_hip_send(ibcomm_hip_comm* comm, int dest_rank, const void* buf, size_t len, int blocking);
+int ibcomm_hip_recv(ibcomm_hip_comm* comm, int src_rank, void* buf, size_t len, int blocking);
+int ibcomm_hip_send_poll(ibcomm_hip_comm* comm, int dest_rank, int* completed);
+int ibcomm_hip_recv_poll(ibcomm_hip_comm* comm, int src_rank, int* completed);
+int ibcomm_hip_send_wait(ibcomm_hip_comm* comm, int dest_rank);
+int ibcomm_hip_recv_wait(ibcomm_hip_comm* comm, int src_rank);
+int ibcomm_hip_bcast(ibcomm_hip_comm* comm, void* buf, size_t len, int root);
+
 /* ---- partitioning and plans (host only, no device needed) ---------------------------------- */
 
 /* IBVerbsCommunicator::SplitBuffer (ibcomm/ibverbs_communicator.cpp:637-683).  env_chunksize is

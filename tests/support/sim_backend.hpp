@@ -286,6 +286,10 @@ struct SimBackend {
     Sim::Get().RunAll();
     return 0;
   }
+  static int CopySync(void* dst, const void* src, size_t bytes) {
+    memmove(dst, src, bytes);
+    return 0;
+  }
   static int CopyAsync(void* dst, const void* src, size_t bytes, Stream s) {
     SimNode n;
     n.kind = 1;

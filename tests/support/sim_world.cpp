@@ -77,6 +77,71 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   return rc;
 }
 
+// Point-to-point scenarios on host buffers; returns a bit per check that held.
+int sim_p2p(void) {
+  Sim::Get().Reset(5);
+  const int world = 4;
+  Fabric<SimBackend> fabric(world);
+  std::vector<std::unique_ptr<Communicator<SimBackend>>> comms;
+  for (int r = 0; r < world; r++) {
+    comms.emplace_back(new Communicator<SimBackend>(&fabric, world));
+    if (comms.back()->Init() != kOk) return -1;
+    comms.back()->RegisterMyself(r);
+  }
+  int held = 0;
+  // ping-pong as in tests/sendrecv_test.cpp: non-blocking Send, blocking Recv, SendWait
+  int value = 10, value2 = -1;
+  bool ok = false;
+  if (comms[0]->Send(1, &value, sizeof value, false) == kOk && comms[1]->Recv(0, &value2, sizeof value2, true) == kOk &&
+      comms[0]->SendWait(1) == kOk && value2 == 10)
+    held |= 1;
+  value2 = -7;
+  if (comms[1]->Send(0, &value2, sizeof value2, false) == kOk && comms[0]->Recv(1, &value, sizeof value, true) == kOk &&
+      comms[1]->SendWait(0) == kOk && value == -7)
+    held |= 2;
+  // a second non-blocking send before SendWait is refused with NOT_SUPPORTED; so is a second Recv
+  int a = 1, b = 2, c = 0, d = 0;
+  if (comms[2]->Send(3, &a, sizeof a, false) == kOk && comms[2]->Send(3, &b, sizeof b, false) == kNotSupported) held |= 4;
+  if (comms[3]->Recv(2, &c, sizeof c, false) == kOk && comms[3]->Recv(2, &d, sizeof d, false) == kNotSupported) held |= 8;
+  // polls: nothing before the data has been moved, exactly one completion afterwards
+  if (comms[2]->SendPoll(3, &ok) == kOk && !ok) held |= 16;
+  if (comms[3]->RecvPoll(2, &ok) == kOk && ok && c == 1 && comms[3]->RecvPoll(2, &ok) == kOk && !ok) held |= 32;
+  if (comms[2]->SendPoll(3, &ok) == kOk && ok && comms[2]->SendPoll(3, &ok) == kOk && !ok) held |= 64;
+  // messages between a pair are delivered in order
+  int seq[3] = {5, 6, 7}, got[3] = {0, 0, 0};
+  bool fifo = true;
+  for (int k = 0; k < 3; k++) {
+    fifo = fifo && comms[0]->Send(2, &seq[k], sizeof(int), false) == kOk && comms[2]->Recv(0, &got[k], sizeof(int), true) == kOk &&
+           comms[0]->SendWait(2) == kOk;
+  }
+  if (fifo && got[0] == 5 && got[1] == 6 && got[2] == 7) held |= 128;
+  // a message larger than the posted buffer is a transport error; bad ranks are invalid arguments
+  long big = 1;
+  char small_buf = 0;
+  if (comms[0]->Send(1, &big, sizeof big, false) == kOk && comms[1]->Recv(0, &small_buf, 1, false) == kOk &&
+      comms[1]->RecvPoll(0, &ok) == kTransportError)
+    held |= 256;
+  if (comms[0]->Send(9, &a, 4, false) == kInvalidArgument && comms[0]->Recv(-1, &a, 4, false) == kInvalidArgument) held |= 512;
+  // broadcast from rank 1 with one thread per rank
+  std::vector<int> vals(world, 0);
+  vals[1] = 4242;
+  Fabric<SimBackend> fabric2(world);
+  std::vector<std::unique_ptr<Communicator<SimBackend>>> c2;
+  for (int r = 0; r < world; r++) {
+    c2.emplace_back(new Communicator<SimBackend>(&fabric2, world));
+    c2.back()->Init();
+    c2.back()->RegisterMyself(r);
+  }
+  std::vector<std::thread> th;
+  std::vector<int> rcs(world, -1);
+  for (int r = 0; r < world; r++) th.emplace_back([&, r]() { rcs[r] = c2[r]->Bcast(&vals[r], sizeof(int), 1); });
+  for (auto& t : th) t.join();
+  bool bc = true;
+  for (int r = 0; r < world; r++) bc = bc && rcs[r] == kOk && vals[r] == 4242;
+  if (bc) held |= 1024;
+  return held;
+}
+
 // Runs one world allreduce with tracing on and dumps rank 0's trace to `path`.
 int sim_trace(int algo, int world, const void* const* sendbufs, void* const* recvbufs, size_t len, int max_fuse,
               const char* path, unsigned long long* pairs /* 7 */) {

@@ -265,3 +265,13 @@ def test_trace_file_has_the_reference_format(tmp_path):
         assert all(d >= 0 for d in durs) and starts == sorted(starts) and all(s >= 0 for s in starts)
         if names[k] in want_pairs:
             assert pairs[k] == want_pairs[names[k]], names[k]
+
+
+def test_point_to_point_over_the_loopback():
+    # Send / Recv / SendPoll / RecvPoll / SendWait / RecvWait / Bcast semantics
+    # (ibcomm/ibverbs_communicator.cpp:371-606, usage as in tests/sendrecv_test.cpp)
+    held = S.lib().sim_p2p()
+    names = ["ping", "pong", "second send refused", "second recv refused", "send not complete before pull",
+             "one recv completion", "one send completion", "fifo", "oversized message", "bad rank", "bcast"]
+    missing = [n for k, n in enumerate(names) if not held >> k & 1]
+    assert not missing, missing

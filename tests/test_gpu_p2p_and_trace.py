@@ -1,0 +1,81 @@
+"""GPU checks of the transport facade (Send/Recv/Poll/Wait/Bcast over the loopback, host and device
+buffers) and of the pipeline trace, through the C ABI."""
+import ctypes as C
+import os
+import threading
+
+import numpy as np
+import pytest
+
+import hip_lib as H
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+import gpu_util as G  # noqa: E402
+
+
+def test_ping_pong_device_and_host_buffers():
+    # tests/sendrecv_test.cpp: non-blocking Send, blocking Recv, then SendWait
+    L = H.lib()
+    with H.World(2) as w:
+        a, b = w.comms
+        src = torch.arange(1000, dtype=torch.int32, device="cuda")
+        dst = torch.zeros(1000, dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
+        assert L.ibcomm_hip_send(a, 1, src.data_ptr(), 4000, 0) == 0
+        assert L.ibcomm_hip_recv(b, 0, dst.data_ptr(), 4000, 1) == 0
+        assert L.ibcomm_hip_send_wait(a, 1) == 0
+        assert torch.equal(src, dst)
+        # device -> host and host -> device
+        host = np.zeros(1000, dtype=np.int32)
+        assert L.ibcomm_hip_send(b, 0, dst.data_ptr(), 4000, 0) == 0
+        assert L.ibcomm_hip_recv(a, 1, host.ctypes.data, 4000, 1) == 0
+        assert L.ibcomm_hip_send_wait(b, 0) == 0
+        assert np.array_equal(host, np.arange(1000, dtype=np.int32))
+        host2 = (host * 3).astype(np.int32)
+        assert L.ibcomm_hip_send(a, 1, host2.ctypes.data, 4000, 0) == 0
+        assert L.ibcomm_hip_send(a, 1, host2.ctypes.data, 4000, 0) == H.NOT_SUPPORTED  # SendWait must come first
+        done = C.c_int(-1)
+        assert L.ibcomm_hip_send_poll(a, 1, C.byref(done)) == 0 and done.value == 0
+        assert L.ibcomm_hip_recv(b, 0, dst.data_ptr(), 4000, 0) == 0
+        assert L.ibcomm_hip_recv_poll(b, 0, C.byref(done)) == 0 and done.value == 1
+        assert L.ibcomm_hip_send_poll(a, 1, C.byref(done)) == 0 and done.value == 1
+        assert np.array_equal(dst.cpu().numpy(), host2)
+
+
+def test_bcast_one_thread_per_rank():
+    L = H.lib()
+    n = 4
+    with H.World(n) as w:
+        bufs = [torch.full((4096,), float(r), device="cuda") for r in range(n)]
+        torch.cuda.synchronize()
+        rcs = [None] * n
+
+        def run(r):
+            rcs[r] = L.ibcomm_hip_bcast(w.comms[r], bufs[r].data_ptr(), 4096 * 4, 2)
+
+        th = [threading.Thread(target=run, args=(r,)) for r in range(n)]
+        [t.start() for t in th]
+        [t.join() for t in th]
+        assert rcs == [0] * n
+        for r in range(n):
+            assert torch.equal(bufs[r], torch.full((4096,), 2.0, device="cuda"))
+
+
+def test_trace_files(tmp_path):
+    base = str(tmp_path / "trace")
+    with G.env(IBCOMM_TRACE_FILE=base, IBCOMM_CHUNKSIZE=None):
+        with H.World(4) as w:
+            w.set_graph_mode(0)
+            w.set_trace(True)
+            send = [torch.randn(1 << 18, device="cuda") for _ in range(4)]
+            recv = [torch.empty_like(t) for t in send]
+            assert G.run_world(w, H.RING, send, recv) == 0
+            w.dump_trace()
+    names = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
+    for r in range(4):
+        lines = open("%s_%d.dat" % (base, r)).read().splitlines()
+        assert [ln.split(",")[0] for ln in lines] == names
+        received = [float(x) for x in lines[0].split(",")[1:-1]]
+        assert len(received) == 2 * 2 * 3 * 4  # (start, duration) x 2(N-1) groups x 4 chunks
+        assert all(d >= 0 for d in received[1::2])
