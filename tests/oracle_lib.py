@@ -168,7 +168,7 @@ def ref_util():
 # Independent numpy statements of what the schedules must compute.  They share
 # no code with the oracle: partitioning is re-derived here from the rule
 # (ibverbs_communicator.cpp:637-707), and sums are explicit numpy adds in the
-# order SURVEY-level analysis of the schedules gives.
+# order that reading the schedules gives (ring: the owner of the chunk group starts; tree: pairwise).
 # --------------------------------------------------------------------------
 
 def np_partition(length, itemsize, world, chunksize=None):

@@ -1,6 +1,6 @@
 """GPU parity of the allreduce engines through the C ABI, bit-exact against the CPU oracle's
 restatement of AllreduceRingCuda / AllreduceRabenseifnerCuda, plus the reference tester's cases
-(tests/allreduce_test.py:102-225) and the BASELINE configurations."""
+(tests/allreduce_test.py:102-225) and the five benchmark configurations at full size."""
 import numpy as np
 import pytest
 
@@ -243,7 +243,7 @@ def test_aging_short():
                 assert all(torch.equal(r, want) for r in recv)
 
 
-# ------------------------------------------------------------------ BASELINE configurations
+# ------------------------------------------------------------------ benchmark configurations, full size
 
 def device_inputs(world_size, n, seed, kind):
     out = []
