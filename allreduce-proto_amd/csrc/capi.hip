@@ -71,8 +71,15 @@ struct ibcomm_hip_fabric {
 
 struct ibcomm_hip_comm {
   ibcomm_hip_comm(ibcomm_hip_fabric* f, int n) : owner(f), comm(&f->fabric, n) {}
+  ~ibcomm_hip_comm() {
+    if (stage_send) (void)hipFree(stage_send);
+    if (stage_recv) (void)hipFree(stage_recv);
+  }
   ibcomm_hip_fabric* owner;
   Communicator<HipBackend> comm;
+  void* stage_send = nullptr;  // device staging for the host-buffer calls, grown on demand
+  void* stage_recv = nullptr;
+  size_t stage_bytes = 0;
 };
 
 struct ibcomm_hip_plan {
@@ -138,6 +145,42 @@ int ibcomm_hip_allreduce_ring(ibcomm_hip_comm* comm, int dtype, const void* send
 int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
   if (!comm) return Fail(kInvalidArgument, "comm is null");
   return comm->comm.AllreduceBlocking(kRabenseifner, dtype, sendbuf, recvbuf, len);
+}
+
+}  // extern "C"
+
+namespace {
+// Host buffers in, host buffers out: copy up, run the device collective, copy down.
+int AllreduceHost(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  const size_t es = DTypeSize(dtype);
+  if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+  if (!sendbuf || !recvbuf) return Fail(kInvalidArgument, "sendbuf and recvbuf must not be null");
+  const size_t bytes = len * es;
+  if (bytes > comm->stage_bytes) {
+    if (comm->stage_send) IBCOMM_HIP_CHECK(hipFree(comm->stage_send));
+    if (comm->stage_recv) IBCOMM_HIP_CHECK(hipFree(comm->stage_recv));
+    comm->stage_send = comm->stage_recv = nullptr;
+    comm->stage_bytes = 0;
+    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_send, bytes));
+    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_recv, bytes));
+    comm->stage_bytes = bytes;
+  }
+  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(comm->stage_send, sendbuf, bytes, hipMemcpyHostToDevice));
+  IBCOMM_RETURN_IF_ERROR(comm->comm.AllreduceBlocking(algo, dtype, comm->stage_send ? comm->stage_send : sendbuf,
+                                                      comm->stage_recv ? comm->stage_recv : recvbuf, len));
+  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(recvbuf, comm->stage_recv, bytes, hipMemcpyDeviceToHost));
+  return kOk;
+}
+}  // namespace
+
+extern "C" {
+
+int ibcomm_hip_allreduce_ring_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return AllreduceHost(comm, kRing, dtype, sendbuf, recvbuf, len);
+}
+int ibcomm_hip_allreduce_rabenseifner_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return AllreduceHost(comm, kRabenseifner, dtype, sendbuf, recvbuf, len);
 }
 
 int ibcomm_hip_allreduce_ring_f32(ibcomm_hip_comm* c, const float* s, float* r, size_t n) {

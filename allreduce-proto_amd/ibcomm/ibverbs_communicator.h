@@ -104,17 +104,15 @@ class IBVerbsCommunicator {
     Check(ibcomm_hip_allreduce_rabenseifner(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
   }
 
-  // The host-buffer variants (ibcomm/allreduce_cpu_impl.h) are the reference's CPU path; this build
-  // accelerates the device path only.
+  // Host buffers (ibcomm/allreduce_cpu_impl.h:23-244, 246-372): staged through the device, same sums in
+  // the same order as the reference's CPU path.
   template <typename T>
-  void AllreduceRing(const T*, T*, size_t) {
-    util::IbcommError(__FILE__, __LINE__, util::IBCOMM_ERROR_CODE::NOT_SUPPORTED,
-                      "AllreduceRing on host buffers is not part of the HIP build; use AllreduceRingCuda.");
+  void AllreduceRing(const T* sendbuf, T* recvbuf, size_t len_elements) {
+    Check(ibcomm_hip_allreduce_ring_host(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
   }
   template <typename T>
-  void AllreduceRabenseifner(const T*, T*, size_t) {
-    util::IbcommError(__FILE__, __LINE__, util::IBCOMM_ERROR_CODE::NOT_SUPPORTED,
-                      "AllreduceRabenseifner on host buffers is not part of the HIP build; use AllreduceRabenseifnerCuda.");
+  void AllreduceRabenseifner(const T* sendbuf, T* recvbuf, size_t len_elements) {
+    Check(ibcomm_hip_allreduce_rabenseifner_host(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
   }
 
   // ibverbs_communicator.cpp:157-216; the trace is recorded when IBCOMM_HIP_TRACE=1.

@@ -21,7 +21,8 @@ LAND_MEMCPY, LAND_KERNEL, LAND_DIRECT = 0, 1, 2
 EXPORTS = [
     "ibcomm_hip_last_error", "ibcomm_hip_fabric_create", "ibcomm_hip_fabric_destroy", "ibcomm_hip_comm_create",
     "ibcomm_hip_comm_destroy", "ibcomm_hip_comm_register_myself", "ibcomm_hip_allreduce_ring",
-    "ibcomm_hip_allreduce_rabenseifner", "ibcomm_hip_allreduce_ring_f32", "ibcomm_hip_allreduce_ring_i32",
+    "ibcomm_hip_allreduce_rabenseifner", "ibcomm_hip_allreduce_ring_host", "ibcomm_hip_allreduce_rabenseifner_host",
+    "ibcomm_hip_allreduce_ring_f32", "ibcomm_hip_allreduce_ring_i32",
     "ibcomm_hip_allreduce_rabenseifner_f32", "ibcomm_hip_allreduce_rabenseifner_i32", "ibcomm_hip_world_allreduce", "ibcomm_hip_world_record", "ibcomm_hip_replay_allreduce",
     "ibcomm_hip_reduce", "ibcomm_hip_reduce_segments", "ibcomm_hip_max_segments", "ibcomm_hip_split_buffer",
     "ibcomm_hip_rank_to_chunk", "ibcomm_hip_get_exp_of_two", "ibcomm_hip_plan_create", "ibcomm_hip_plan_destroy",
@@ -61,6 +62,7 @@ def lib():
     L.ibcomm_hip_comm_register_myself.argtypes = [vp, i]
     for name in ("ibcomm_hip_allreduce_ring", "ibcomm_hip_allreduce_rabenseifner"):
         getattr(L, name).argtypes = [vp, i, vp, vp, sz]
+        getattr(L, name + "_host").argtypes = [vp, i, vp, vp, sz]
         for suffix in ("_f32", "_i32"):
             getattr(L, name + suffix).argtypes = [vp, vp, vp, sz]
     L.ibcomm_hip_world_allreduce.argtypes = [C.POINTER(vp), i, i, i, C.POINTER(vp), C.POINTER(vp), sz]
@@ -206,11 +208,15 @@ class World:
         """`rank` alone against the recorded peers."""
         return lib().ibcomm_hip_replay_allreduce(self.comms[rank], algo, dtype, send_ptr, recv_ptr, length)
 
-    def allreduce_threads(self, algo, dtype, send_ptrs, recv_ptrs, length):
-        """One host thread per rank, each in the blocking per-rank call (how the reference is used)."""
+    def allreduce_threads(self, algo, dtype, send_ptrs, recv_ptrs, length, host=False):
+        """One host thread per rank, each in the blocking per-rank call (how the reference is used).
+        With host=True the pointers are host memory (the AllreduceRing / AllreduceRabenseifner calls)."""
         import threading
         L = lib()
-        fn = L.ibcomm_hip_allreduce_ring if algo == RING else L.ibcomm_hip_allreduce_rabenseifner
+        if host:
+            fn = L.ibcomm_hip_allreduce_ring_host if algo == RING else L.ibcomm_hip_allreduce_rabenseifner_host
+        else:
+            fn = L.ibcomm_hip_allreduce_ring if algo == RING else L.ibcomm_hip_allreduce_rabenseifner
         rcs = [None] * self.n
         msgs = [""] * self.n
 

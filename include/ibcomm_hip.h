@@ -87,7 +87,19 @@ int ibcomm_hip_allreduce_ring(ibcomm_hip_comm* comm, int dtype, const void* send
 int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
                                       size_t len_elements);
 
-/* Typed spellings of the two calls above, one per template instantiation the reference's own
+/* IBVerbsCommunicator::AllreduceRing<T> and AllreduceRabenseifner<T> on HOST buffers
+ * (ibcomm/allreduce_cpu_impl.h:23-244, 246-372).  The reference computes these on the CPU; here
+ * the data is copied to the device, reduced by the device path above and copied back.  The sums and
+ * their order are the same (ring: left fold from the owner of the chunk group under
+ * SplitBuffer; Rabenseifner: balanced tree, which does not depend on how the buffer is cut), so the
+ * results are bit-identical to the reference's.  One difference: the reference's CPU Rabenseifner does
+ * not go through SplitBuffer and therefore accepts len_elements < world_size, which returns 4 here. */
+int ibcomm_hip_allreduce_ring_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
+                                   size_t len_elements);
+int ibcomm_hip_allreduce_rabenseifner_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
+                                           size_t len_elements);
+
+/* Typed spellings of the two device-buffer calls, one per template instantiation the reference's own
  * programs use. */
 int ibcomm_hip_allreduce_ring_f32(ibcomm_hip_comm* comm, const float* sendbuf, float* recvbuf, size_t len_elements);
 int ibcomm_hip_allreduce_ring_i32(ibcomm_hip_comm* comm, const int32_t* sendbuf, int32_t* recvbuf, size_t len_elements);

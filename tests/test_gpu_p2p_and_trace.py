@@ -79,3 +79,22 @@ def test_trace_files(tmp_path):
         received = [float(x) for x in lines[0].split(",")[1:-1]]
         assert len(received) == 2 * 2 * 3 * 4  # (start, duration) x 2(N-1) groups x 4 chunks
         assert all(d >= 0 for d in received[1::2])
+
+
+@pytest.mark.parametrize("algo,oracle_algo,world_size", [(H.RING, 0, 4), (H.RING, 0, 3), (H.RABENSEIFNER, 1, 4), (H.RABENSEIFNER, 1, 8)])
+def test_host_buffer_calls_match_the_reference_cpu_path(algo, oracle_algo, world_size):
+    # AllreduceRing<T> / AllreduceRabenseifner<T> on host memory (ibcomm/allreduce_cpu_impl.h), bit-exact
+    # against the oracle's restatement of those CPU routines (O.RING_CPU = 0, O.RABEN_CPU = 1)
+    import oracle_lib as O
+    n = 100003 if algo == H.RING else 8 * 12500 + 3 * world_size  # the CPU Rabenseifner needs ceil(n/N)*(N-1) <= n
+    host = [np.random.default_rng(50 + r).standard_normal(n).astype(np.float32) for r in range(world_size)]
+    orc, want, _ = O.allreduce(oracle_algo, host)
+    assert orc == 0
+    out = [np.full(n, 7.0, dtype=np.float32) for _ in range(world_size)]
+    with G.env(IBCOMM_CHUNKSIZE=None):
+        with H.World(world_size) as w:
+            for _ in range(2):
+                rcs, msgs = w.allreduce_threads(algo, H.F32, [h.ctypes.data for h in host], [o.ctypes.data for o in out], n, host=True)
+                assert rcs == [0] * world_size, msgs
+                for r in range(world_size):
+                    assert np.array_equal(O.bits(out[r]), O.bits(want[r])), "rank %d" % r
