@@ -220,21 +220,25 @@ def main():
     sp = [t.data_ptr() for t in send]
     rp = [t.data_ptr() for t in recv]
 
+    # Shape of the dominant reduction launch of rank 0, from its plan: one ring step reduces one chunk
+    # group; the first Rabenseifner halving step reduces half of all groups (the largest window).
+    p = H.Plan(algo, world, 0, n, 4, chunk)
+    fuse = args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64"))
+    if algo == H.RING:
+        per_step = len(p.ranges) // world
+    else:
+        per_step = sum(1 for _, peer, kind in p.recvs if kind == 0)
+    leg_segments = max(1, min(fuse, per_step))
+    seg_elems = p.ranges[0][1] - p.ranges[0][0]
+
     if args.only_roofline:
-        p = H.Plan(algo, world, 0, n, 4, chunk)
-        fuse = args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64"))
-        if algo == H.RING:
-            per_step = len(p.ranges) // world            # one ring step reduces one group
-        else:
-            per_step = sum(1 for _, peer, kind in p.recvs if kind == 0)  # the first halving step's window
-        seg_elems = p.ranges[0][1] - p.ranges[0][0]
         # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
         # counters collected over this command can be calibrated against a known traffic
         for _ in range(3):
             recv[0].copy_(send[0])
         torch.cuda.synchronize()
         print(json.dumps({"only_roofline": True, "config": args.config,
-                          "roofline": roofline_leg(torch, H, send, recv, seg_elems, max(1, min(fuse, per_step)), 200)}))
+                          "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)}))
         return
 
     def timed(call, steps, warm):
@@ -283,9 +287,7 @@ def main():
 
     rank_bytes = device_bytes(st_rank)
     world_bytes = sum(device_bytes(s) for s in st)
-    segs_per_launch = max(1, round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"])))
-    first = H.Plan(algo, world, rank, n, 4, chunk).ranges[0]
-    seg_elems = first[1] - first[0]
+    segs_per_launch = round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"]), 2)
 
     algbw = n * 4 / sec_per_step * 1e-9
     world_algbw = n * 4 / world_sec * 1e-9
@@ -318,7 +320,7 @@ def main():
             "rank_device_GBps": round(rank_bytes / sec_per_step * 1e-9, 1),
             "rank_frac_of_hbm_peak": round(rank_bytes / sec_per_step * 1e-9 / HBM_PEAK_GBPS, 4),
             "rank_reduce_launches_per_step": st_rank["reduce_launches"],
-            "rank_segments_per_launch": segs_per_launch,
+            "rank_mean_segments_per_launch": segs_per_launch,
             "rank_reduce_elements_per_step": st_rank["reduce_elements"],
             "rank_landing_launches_per_step": st_rank["landing_copies"],
             "rank_gather_launches_per_step": st_rank["gather_copies"],
@@ -336,7 +338,7 @@ def main():
         },
     }
     if not args.no_roofline:
-        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, 200)
+        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
     del recv
     if not args.no_cpu:
         del send
