@@ -282,6 +282,19 @@ def main():
         world_sec = timed(lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), args.steps, warm)
         graph_counters = w.graph_counters()
 
+        # 4. for reference: the same single-rank schedule with zero-copy landing (the reduction reads each
+        #    message where it lies instead of from a pool slot), unless that is the mode already measured
+        direct = None
+        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "kernel")) != "direct":
+            w.set_landing(H.LAND_DIRECT)
+            out = torch.empty_like(send[rank])
+            direct_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
+            direct_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
+            parity = parity and direct_ok
+            direct = {"ms_per_step": round(direct_sec * 1e3, 4), "algbw_GBps": round(n * 4 / direct_sec * 1e-9, 2),
+                      "parity_bit_exact": direct_ok}
+            del out
+
     def device_bytes(s):
         return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
 
@@ -331,6 +344,7 @@ def main():
                 "device_GBps": round(world_bytes / world_sec * 1e-9, 1),
                 "frac_of_hbm_peak": round(world_bytes / world_sec * 1e-9 / HBM_PEAK_GBPS, 4),
             },
+            "rank_zero_copy_landing": direct,
             "streams_per_rank": st[0]["streams_created"],
             "issue": "eager" if args.no_graph else "hip graph replay",
             "graph_calls_eager_captured_replayed": list(graph_counters),
