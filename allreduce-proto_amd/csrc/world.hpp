@@ -97,17 +97,20 @@ int RunAlone(Communicator<B>* comm, int algo, int dtype, const void* sendbuf, vo
     const int rc = comm->Progress(&progressed, &finished);
     if (rc != kOk) {
       comm->Abort();
+      comm->fabric()->Reset();  // completions of sends to the ghosts must not leak into the next call
       return rc;
     }
     if (finished) break;
     if (!progressed) {
       comm->Abort();
+      comm->fabric()->Reset();
       return Fail(kTransportError, "replay of rank %d stalled at receive %zu/%zu, send %zu/%zu: the recording is of a different call",
                   comm->rank(), comm->recv_cursor(), comm->recv_total(), comm->send_cursor(), comm->send_total());
     }
   }
   if (!comm->fabric()->ReplayDrained()) {
     comm->Abort();
+    comm->fabric()->Reset();
     return Fail(kTransportError, "replay of rank %d left recorded messages unused: the recording is of a different call", comm->rank());
   }
   if (synchronize) return comm->Finish(false);

@@ -77,6 +77,90 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   return rc;
 }
 
+// Failure handling, forced from the host; returns a bit per check that held.
+int sim_failures(void) {
+  Sim::Get().Reset(9);
+  int held = 0;
+  std::vector<float> a(4096, 1.0f), b(4096, 2.0f), ra(4096), rb(4096);
+  {
+    // a rank whose peer never shows up gives up after IBCOMM_HIP_TIMEOUT_S with a transport error
+    Fabric<SimBackend> fabric(2);
+    Communicator<SimBackend> c0(&fabric, 2), c1(&fabric, 2);
+    c0.Init(); c1.Init();
+    c0.RegisterMyself(0); c1.RegisterMyself(1);
+    setenv("IBCOMM_HIP_TIMEOUT_S", "0.2", 1);
+    const int rc = c0.AllreduceBlocking(kRing, kF32, a.data(), ra.data(), a.size());
+    unsetenv("IBCOMM_HIP_TIMEOUT_S");
+    if (rc == kTransportError && !c0.active()) held |= 1;
+    fabric.Reset();
+    // ... and the communicator is usable afterwards
+    const void* sends[2] = {a.data(), b.data()};
+    void* recvs[2] = {ra.data(), rb.data()};
+    Communicator<SimBackend>* cs[2] = {&c0, &c1};
+    if (RunWorld<SimBackend>(cs, 2, kRing, kF32, sends, recvs, a.size(), true) == kOk && ra[7] == 3.0f && rb[4095] == 3.0f) held |= 2;
+  }
+  {
+    // ranks that disagree about the buffer length: the first mismatching message is a transport error
+    Fabric<SimBackend> fabric(2);
+    Communicator<SimBackend> c0(&fabric, 2), c1(&fabric, 2);
+    c0.Init(); c1.Init();
+    c0.RegisterMyself(0); c1.RegisterMyself(1);
+    int rc = c0.Begin(kRing, kF32, a.data(), ra.data(), 4096);
+    if (rc == kOk) rc = c1.Begin(kRing, kF32, b.data(), rb.data(), 2048);
+    bool p = false, f = false;
+    int r0 = kOk, r1 = kOk;
+    for (int k = 0; k < 8 && r0 == kOk && r1 == kOk; k++) {
+      r0 = c0.Progress(&p, &f);
+      if (r0 == kOk) r1 = c1.Progress(&p, &f);
+    }
+    if (rc == kOk && (r0 == kTransportError || r1 == kTransportError)) held |= 4;
+    c0.Abort(); c1.Abort();
+  }
+  {
+    // a second collective on a communicator that is still inside one is refused (NOT_SUPPORTED)
+    Fabric<SimBackend> fabric(2);
+    Communicator<SimBackend> c0(&fabric, 2);
+    c0.Init(); c0.RegisterMyself(0);
+    if (c0.Begin(kRing, kF32, a.data(), ra.data(), 4096) == kOk &&
+        c0.Begin(kRing, kF32, a.data(), ra.data(), 4096) == kNotSupported) held |= 8;
+    // point-to-point calls are refused while it runs
+    if (c0.Send(1, a.data(), 4, false) == kNotSupported) held |= 16;
+    c0.Abort();
+    // partially overlapping buffers and null pointers are invalid arguments
+    if (c0.Begin(kRing, kF32, a.data(), a.data() + 8, 2048) == kInvalidArgument &&
+        c0.Begin(kRing, kF32, nullptr, ra.data(), 2048) == kInvalidArgument &&
+        c0.Begin(kRing, 99, a.data(), ra.data(), 2048) == kInvalidArgument) held |= 32;
+  }
+  {
+    // a replay needs a recording of the same rank and the same call
+    Fabric<SimBackend> fabric(2);
+    Communicator<SimBackend> c0(&fabric, 2), c1(&fabric, 2);
+    c0.Init(); c1.Init();
+    c0.RegisterMyself(0); c1.RegisterMyself(1);
+    Communicator<SimBackend>* cs[2] = {&c0, &c1};
+    const void* sends[2] = {a.data(), b.data()};
+    void* recvs[2] = {ra.data(), rb.data()};
+    if (!fabric.StartReplay(0)) held |= 64;  // nothing recorded yet
+    size_t bytes = 0;
+    c0.RecordingBytes(kRing, kF32, 4096, &bytes);
+    fabric.StartRecording(0, bytes);
+    int rc = RunWorld<SimBackend>(cs, 2, kRing, kF32, sends, recvs, 4096, true);
+    fabric.StopRecording();
+    if (rc == kOk && !fabric.StartReplay(1)) held |= 128;  // recorded rank 0, not rank 1
+    if (fabric.StartReplay(0)) {
+      std::vector<float> out(4096);
+      // a different length: the first recorded message does not fit the plan
+      rc = RunAlone<SimBackend>(&c0, kRing, kF32, a.data(), out.data(), 2048, true);
+      if (rc == kTransportError && !c0.active()) held |= 256;
+      // the right call still replays afterwards
+      rc = RunAlone<SimBackend>(&c0, kRing, kF32, a.data(), out.data(), 4096, true);
+      if (rc == kOk && out[100] == 3.0f) held |= 512;
+      fabric.StopReplay();
+    }
+  }
+  return held;
+}
+
 // Point-to-point scenarios on host buffers; returns a bit per check that held.
 int sim_p2p(void) {
   Sim::Get().Reset(5);

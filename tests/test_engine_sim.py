@@ -275,3 +275,14 @@ def test_point_to_point_over_the_loopback():
              "one recv completion", "one send completion", "fifo", "oversized message", "bad rank", "bcast"]
     missing = [n for k, n in enumerate(names) if not held >> k & 1]
     assert not missing, missing
+
+
+def test_failure_handling_is_reported_not_hung():
+    # a missing peer, disagreeing ranks, re-entrancy, bad arguments and a mismatched replay all come
+    # back as the reference's error codes, and the communicators stay usable
+    held = S.lib().sim_failures()
+    names = ["missing peer times out", "usable after a timeout", "length mismatch", "second collective refused",
+             "p2p refused during a collective", "bad arguments", "replay without recording", "replay of another rank",
+             "replay of another call", "replay still works"]
+    missing = [n for k, n in enumerate(names) if not held >> k & 1]
+    assert not missing, missing
