@@ -159,7 +159,7 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     bufs = [np.random.default_rng(900 + r).standard_normal(n).astype(np.float32) for r in range(world)]
     algo = O.RING_CPU if algo_name == "ring" else O.RABEN_CPU
     times = []
-    for i in range(3):  # 1 warm-up + 2 timed
+    for i in range(6):  # 1 warm-up + 5 timed
         t0 = time.perf_counter()
         rc, recv, _ = O.allreduce(algo, bufs, chunk if algo_name == "ring" else None)
         t1 = time.perf_counter()
@@ -168,16 +168,18 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
             times.append(t1 - t0)
         del recv
     t = min(times)
-    single = O.lib().orc_time_reduce_f32(16 * 1024 * 1024, 5)
+    single_n = 64 * 1024 * 1024  # 256 MiB per operand: memory-bound on any host
+    single = O.lib().orc_time_reduce_f32(single_n, 3)
     return {
         "value": round(n * 4 / t * 1e-9, 3),
         "unit": "GB/s algbw",
         "cores": min(world, os.cpu_count() or 1),
         "kind": "port",
-        "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 2 after 1 warm-up, "
+        "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 5 after 1 warm-up, "
                   "one host thread per emulated rank on %d logical CPUs" % (algo_name, world, n, chunk, os.cpu_count() or 1),
         "seconds": round(t, 3),
-        "single_core_reduce_loop_GBps": round(12.0 * 16 * 1024 * 1024 / single * 1e-9, 2),
+        "seconds_median": round(sorted(times)[len(times) // 2], 3),
+        "single_core_reduce_loop_GBps": round(12.0 * single_n / single * 1e-9, 2),
     }
 
 
