@@ -355,6 +355,10 @@ def main():
     }
     if not args.no_roofline:
         line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+        # the same kernel over one whole per-rank buffer: what it sustains once the launch is large
+        whole = roofline_leg(torch, H, send, recv, n, 1, 40)
+        line["roofline"]["whole_buffer_launch"] = {k: whole[k] for k in (
+            "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
     del recv
     if not args.no_cpu:
         del send

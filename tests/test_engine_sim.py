@@ -286,3 +286,34 @@ def test_failure_handling_is_reported_not_hung():
              "replay of another call", "replay still works"]
     missing = [n for k, n in enumerate(names) if not held >> k & 1]
     assert not missing, missing
+
+
+def test_randomised_shapes_and_knobs():
+    # random worlds, lengths, chunk sizes, fusion limits, landing modes, stream counts and schedules;
+    # every case must be bit-identical to the oracle and free of unordered conflicting accesses
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        algo = int(rng.integers(0, 2))
+        world = int(rng.choice([2, 4, 8, 16])) if algo == RABEN else int(rng.integers(2, 10))
+        n = int(rng.integers(world, 6000))
+        chunk = None
+        if rng.random() < 0.6:
+            epc = int(rng.integers(1, max(2, n // (2 * world) + 1)))
+            if -(-n // epc) >= 2 * world:
+                chunk = 4 * epc
+        dtype = [np.float32, np.int32, np.float64][int(rng.integers(0, 3))]
+        if chunk is not None and dtype == np.float64:
+            chunk *= 2
+        bufs = [(np.random.default_rng(case * 100 + r).standard_normal(n) * 50).astype(dtype) for r in range(world)]
+        kw = dict(max_fuse=int(rng.integers(1, 65)), landing=int(rng.integers(0, 3)), seed=case,
+                  streams=int(rng.integers(1, 9)), pool_bytes=int(rng.choice([512, 4096, 65536])),
+                  in_place=bool(rng.random() < 0.2), threaded=bool(rng.random() < 0.15))
+        orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs, chunk)
+        assert orc == 0, (case, algo, world, n, chunk)
+        rc, recv, rep = S.allreduce(algo, bufs, chunk, **kw)
+        assert rc == 0, (case, rep.error.decode(), algo, world, n, chunk, kw)
+        for r in range(world):
+            assert np.array_equal(O.bits(recv[r]), O.bits(want[r])), (case, r, algo, world, n, chunk, kw)
+        assert rep.unrecorded_waits == 0
+        if not kw["threaded"]:
+            assert rep.races == 0, (case, rep.first_race.decode(), kw)
