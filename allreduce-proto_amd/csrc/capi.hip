@@ -499,7 +499,7 @@ int ibcomm_hip_comm_set_max_fuse(ibcomm_hip_comm* comm, int f) {
 
 int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode) {
   if (!comm) return Fail(kInvalidArgument, "comm is null");
-  if (mode < kLandMemcpy || mode > kLandDirect) return Fail(kInvalidArgument, "landing mode must be 0, 1 or 2");
+  if (mode < kLandMemcpy || mode > kLandStaged) return Fail(kInvalidArgument, "landing mode must be 0, 1, 2 or 3");
   comm->comm.set_landing(mode);
   return kOk;
 }

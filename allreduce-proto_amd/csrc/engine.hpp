@@ -10,14 +10,19 @@
 //     this rank consumes and emits;
 //   * Progress() walks the plan without ever waiting for the device: it posts
 //     every send whose data has been *enqueued*, takes every message a peer
-//     has posted, lands it in a pool slot (one copy-kernel launch for all of
-//     them by default, or one hipMemcpyAsync each), and launches one segment
-//     kernel over all chunks that landed in this pass:
-//         recvbuf[c] = incoming + sendbuf[c]     ring steps, first halving step
-//         recvbuf[c] = incoming + recvbuf[c]     later halving steps
-//     Finished chunks of the gather phase land straight in recvbuf and are
-//     forwarded from there, so they cost one copy instead of the reference's
-//     three (:129-135, :528-529);
+//     has posted, and launches one segment kernel over all chunks taken in
+//     this pass:
+//         result[c] = incoming + sendbuf[c]     ring steps, first halving step
+//         result[c] = incoming + recvbuf[c]     later halving steps
+//     By default ("staged") the kernel reads the incoming partial sum where
+//     the sender staged it, and writes result[c] into a pool slot of its own
+//     when the sum is only going to be forwarded, into recvbuf when this rank
+//     keeps it: the reference's copy to the staging slot (:134-135, :515-516)
+//     is the kernel's store.  The other modes first land each message in a
+//     local pool slot, by one copy-kernel launch per pass or one
+//     hipMemcpyAsync per message.  Finished chunks of the gather phase land
+//     straight in recvbuf and are forwarded from there, so they cost one copy
+//     instead of the reference's three (:129-135, :528-529);
 //   * ordering between ranks, streams and slot reuse is carried by events, so
 //     the same sequence of calls can be recorded into a graph.
 //
@@ -52,6 +57,8 @@ enum LandingMode : int {
   kLandMemcpy = 0,  // one asynchronous device copy per message into a pool slot
   kLandKernel = 1,  // all messages of a pass land through one copy-kernel launch
   kLandDirect = 2,  // no landing: the reduction reads the sender's buffer in place
+  kLandStaged = 3,  // like direct, and a partial sum that is only forwarded is written by the reduction
+                    // into a pool slot (send staging) instead of recvbuf; the next rank reads it there
 };
 
 struct EngineStats {
@@ -101,10 +108,11 @@ class Communicator {
     if (max_fuse_ < 1 || max_fuse_ > kMaxSegments)
       return Fail(kInvalidArgument, "IBCOMM_HIP_MAX_FUSE must be in [1, %d]", kMaxSegments);
     v = getenv("IBCOMM_HIP_LANDING");
-    if (!v || !strcmp(v, "kernel")) landing_ = kLandKernel;
+    if (!v || !strcmp(v, "staged")) landing_ = kLandStaged;
+    else if (!strcmp(v, "kernel")) landing_ = kLandKernel;
     else if (!strcmp(v, "memcpy")) landing_ = kLandMemcpy;
     else if (!strcmp(v, "direct")) landing_ = kLandDirect;
-    else return Fail(kInvalidArgument, "IBCOMM_HIP_LANDING must be memcpy, kernel or direct, not '%s'", v);
+    else return Fail(kInvalidArgument, "IBCOMM_HIP_LANDING must be memcpy, kernel, direct or staged, not '%s'", v);
     // The working GPU buffer (IBCOMM_WORK_GPU_MEMORY_SIZE, ibverbs_communicator_cuda.cpp:12-33) held
     // the second operand of the Rabenseifner kernel.  Here that kernel reads the pool slot itself,
     // so no such buffer is allocated; the variable is still accepted so job scripts keep working.
@@ -190,6 +198,7 @@ class Communicator {
 
     const size_t chunks = plan_.part.ranges.size();
     recv_done_.assign(plan_.recvs.size(), OpState());
+    staged_.assign(plan_.recvs.size(), nullptr);
     chunk_last_.assign(chunks, OpState());
     chunk_unconsumed_.assign(chunks, 0);
     chunk_pulled_.assign(chunks, OpState());
@@ -379,6 +388,8 @@ class Communicator {
     bool active = false;
   };
 
+  bool ZeroCopyReceive() const { return landing_ == kLandDirect || landing_ == kLandStaged; }
+
   char* RecvPtr(int chunk) const { return recvbuf_ + plan_.part.ranges[chunk].begin * es_; }
   const char* SendPtr(int chunk) const { return sendbuf_ + plan_.part.ranges[chunk].begin * es_; }
   size_t ChunkElems(int chunk) const { return plan_.part.ranges[chunk].size(); }
@@ -431,7 +442,12 @@ class Communicator {
         const SendOp& s = plan_.sends[ps.send_index];
         outstanding_sends_--;
         if (c.has_done) pull_events_.push_back(c.done);
-        if (s.dep >= 0 || in_place_) {
+        if (s.dep >= 0 && staged_[s.dep] != nullptr) {
+          // the peer has fetched the staged partial sum: the slot is free once its read completes
+          if (c.has_done) controller_.returnMemory(staged_[s.dep], c.done, c.done_stream);
+          else controller_.returnMemory(staged_[s.dep]);
+          staged_[s.dep] = nullptr;
+        } else if (s.dep >= 0 || in_place_) {
           chunk_unconsumed_[s.chunk]--;
           OpState& p = chunk_pulled_[s.chunk];
           p.issued = true;
@@ -457,7 +473,7 @@ class Communicator {
       } else {
         const OpState& d = recv_done_[s.dep];
         if (!d.issued) break;  // the data has not been enqueued yet
-        src = RecvPtr(s.chunk);
+        src = staged_[s.dep] ? staged_[s.dep]->LandingFor(RecvPtr(s.chunk)) : RecvPtr(s.chunk);
         ready = d.event;
         ready_stream = d.stream;
         has_ready = d.has_event;
@@ -465,7 +481,8 @@ class Communicator {
       TraceScope scope(&trace_, Trace::kIssueSend);
       const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready, ready_stream);
       posted_[s.peer].push_back(PostedSend{ticket, static_cast<int>(next_send_)});
-      if (s.dep >= 0 || in_place_) chunk_unconsumed_[s.chunk]++;
+      const bool from_staging = s.dep >= 0 && staged_[s.dep] != nullptr;
+      if (!from_staging && (s.dep >= 0 || in_place_)) chunk_unconsumed_[s.chunk]++;
       outstanding_sends_++;
       stats_.messages_sent++;
       next_send_++;
@@ -500,9 +517,10 @@ class Communicator {
         // Segments of one launch run concurrently: a chunk whose previous partial sum is still
         // waiting in this batch must go into the next launch.
         if (chunk_in_batch_[r.chunk]) IBCOMM_RETURN_IF_ERROR(FlushReduces());
-        if (landing_ != kLandDirect) {
+        {
+          // One entry per partial sum accepted, whether or not it needs a landing slot of its own.
           TraceScope scope(&trace_, Trace::kIssueRecv);
-          IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+          if (!ZeroCopyReceive()) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
         }
         chunk_in_batch_[r.chunk] = 1;
         pending_reduce_.push_back(p);
@@ -627,7 +645,7 @@ class Communicator {
       const PendingRecv& p = pending_reduce_[i];
       const RecvOp& r = plan_.recvs[p.op];
       const int c = r.chunk;
-      const void* incoming = (landing_ == kLandDirect) ? p.msg.src : p.slot->LandingFor(RecvPtr(c));
+      const void* incoming = ZeroCopyReceive() ? p.msg.src : p.slot->LandingFor(RecvPtr(c));
       const void* own;
       if (r.kind == kReduceWithSendbuf) {
         own = SendPtr(c);
@@ -635,7 +653,16 @@ class Communicator {
         own = RecvPtr(c);
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));  // the previous halving step's sum
       }
-      batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, incoming, own, ChunkElems(c)};
+      void* result = RecvPtr(c);
+      if (landing_ == kLandStaged && plan_.forward_only[p.op] >= 0) {
+        // Nobody on this rank reads this partial sum: produce it where the next rank will fetch it.
+        Memory<B>* stage = nullptr;
+        IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&stage));
+        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, stage));
+        staged_[p.op] = stage;
+        result = stage->LandingFor(RecvPtr(c));
+      }
+      batch.seg[batch.count++] = Segment{result, nullptr, incoming, own, ChunkElems(c)};
       stats_.reduce_elements += ChunkElems(c);
     }
     IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 0));
@@ -651,7 +678,7 @@ class Communicator {
       recv_done_[p.op] = done;
       chunk_last_[r.chunk] = done;
       if (p.slot) controller_.returnMemory(p.slot, done.event, s);
-      if (landing_ == kLandDirect) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
+      if (ZeroCopyReceive()) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
       chunk_in_batch_[r.chunk] = 0;
     }
     pending_reduce_.clear();
@@ -702,7 +729,7 @@ class Communicator {
   MemoryPool<B> pool_;
   MemoryController<B> controller_;
   int max_fuse_ = kMaxSegments;
-  int landing_ = kLandKernel;
+  int landing_ = kLandStaged;
   long long work_gpu_memory_size_ = 0;
 
   bool active_ = false;
@@ -716,6 +743,7 @@ class Communicator {
   size_t next_send_ = 0, next_recv_ = 0;
   size_t outstanding_sends_ = 0;
   std::vector<OpState> recv_done_;        // per receive op: result enqueued (+ completion event)
+  std::vector<Memory<B>*> staged_;        // per receive op: the send-staging slot holding its result, if any
   std::vector<OpState> chunk_last_;       // per chunk: our last device op that wrote recvbuf[chunk]
   std::vector<int> chunk_unconsumed_;     // per chunk: our sends out of recvbuf[chunk] no peer has taken yet
   std::vector<OpState> chunk_pulled_;     // per chunk: the peer's latest read of recvbuf[chunk]

@@ -51,7 +51,37 @@ struct Plan {
   Partition part;
   std::vector<RecvOp> recvs;
   std::vector<SendOp> sends;
+  // Per receive: the one send that forwards its result when that result is needed nowhere else on
+  // this rank (a later gather overwrites the chunk), else -1.  Such a partial sum may be produced
+  // straight into send staging instead of recvbuf.
+  std::vector<int> forward_only;
 };
+
+namespace detail {
+
+inline void MarkForwardOnly(Plan* plan) {
+  const size_t n = plan->recvs.size();
+  plan->forward_only.assign(n, -1);
+  std::vector<int> sends_of(n, 0), send_index(n, -1);
+  for (size_t k = 0; k < plan->sends.size(); k++) {
+    const int d = plan->sends[k].dep;
+    if (d >= 0) {
+      sends_of[d]++;
+      send_index[d] = static_cast<int>(k);
+    }
+  }
+  std::vector<char> gathered_later(plan->part.ranges.size(), 0);
+  for (size_t j = n; j-- > 0;) {
+    const RecvOp& r = plan->recvs[j];
+    if (r.kind == kGather) {
+      gathered_later[r.chunk] = 1;
+    } else if (gathered_later[r.chunk] && sends_of[j] == 1) {
+      plan->forward_only[j] = send_index[j];
+    }
+  }
+}
+
+}  // namespace detail
 
 namespace detail {
 
@@ -169,6 +199,7 @@ inline int BuildPlan(int algo, int world_size, int rank, size_t len_elements, si
   plan->recvs.clear();
   plan->sends.clear();
   if (world_size < 1 || rank < 0 || rank >= world_size) return Fail(kInvalidArgument, "rank %d outside world of %d", rank, world_size);
+  plan->forward_only.clear();
   if (world_size == 1) {
     plan->part = Partition();
     return kOk;
@@ -180,6 +211,7 @@ inline int BuildPlan(int algo, int world_size, int rank, size_t len_elements, si
   if (algo == kRing) BuildRingPlan(world_size, rank, plan);
   else if (algo == kRabenseifner) BuildRabenseifnerPlan(world_size, rank, plan);
   else return Fail(kInvalidArgument, "unknown algorithm %d", algo);
+  detail::MarkForwardOnly(plan);
   return kOk;
 }
 

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(HERE, "libibcomm_hip.so")
 OK, INVALID_ARGUMENT, TRANSPORT_ERROR, DEVICE_ERROR, NOT_SUPPORTED = 0, 1, 2, 3, 4
 F32, I32, F64, I64 = 0, 1, 2, 3
 RING, RABENSEIFNER = 0, 1
-LAND_MEMCPY, LAND_KERNEL, LAND_DIRECT = 0, 1, 2
+LAND_MEMCPY, LAND_KERNEL, LAND_DIRECT, LAND_STAGED = 0, 1, 2, 3
 
 EXPORTS = [
     "ibcomm_hip_last_error", "ibcomm_hip_fabric_create", "ibcomm_hip_fabric_destroy", "ibcomm_hip_comm_create",

@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
 
 One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
-collective: every message the rank receives is landed in its HBM pool, reduced into recvbuf or
-gathered, exactly as in the full world.  The other emulated ranks are replaced by a recording of
+collective: every partial sum the rank receives is added to its own contribution (the result going
+to a pool slot for forwarding, or to recvbuf), every finished chunk is gathered into recvbuf,
+exactly as in the full world.  The other emulated ranks are replaced by a recording of
 what they sent (made by first running the whole world once, all sendbufs resident in HBM), paced
 the way the real dependency on upstream ranks paces them.  The headline `value` is the allreduce
 algorithm bandwidth of that schedule, len * 4 B / time per step.  `extra.world_all_ranks_on_one_gpu`
@@ -189,7 +190,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
-    ap.add_argument("--landing", choices=["memcpy", "kernel", "direct"], default=None)
+    ap.add_argument("--landing", choices=["memcpy", "kernel", "direct", "staged"], default=None)
     ap.add_argument("--fuse", type=int, default=None)
     ap.add_argument("--no-graph", action="store_true", help="issue every step eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -257,7 +258,7 @@ def main():
     rank = 0
     with H.World(world) as w:
         if args.landing:
-            w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT}[args.landing])
+            w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT, "staged": H.LAND_STAGED}[args.landing])
         if args.fuse:
             w.set_max_fuse(args.fuse)
         if args.no_graph:
@@ -284,17 +285,17 @@ def main():
         world_sec = timed(lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), args.steps, warm)
         graph_counters = w.graph_counters()
 
-        # 4. for reference: the same single-rank schedule with zero-copy landing (the reduction reads each
-        #    message where it lies instead of from a pool slot), unless that is the mode already measured
-        direct = None
-        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "kernel")) != "direct":
-            w.set_landing(H.LAND_DIRECT)
+        # 4. for reference: the same single-rank schedule when every message is first copied into a pool
+        #    slot of the receiver by a copy kernel ("kernel" landing), unless that is the mode already measured
+        copied = None
+        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")) != "kernel":
+            w.set_landing(H.LAND_KERNEL)
             out = torch.empty_like(send[rank])
-            direct_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
-            direct_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
-            parity = parity and direct_ok
-            direct = {"ms_per_step": round(direct_sec * 1e3, 4), "algbw_GBps": round(n * 4 / direct_sec * 1e-9, 2),
-                      "parity_bit_exact": direct_ok}
+            copied_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
+            copied_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
+            parity = parity and copied_ok
+            copied = {"ms_per_step": round(copied_sec * 1e3, 4), "algbw_GBps": round(n * 4 / copied_sec * 1e-9, 2),
+                      "parity_bit_exact": copied_ok}
             del out
 
     def device_bytes(s):
@@ -325,7 +326,7 @@ def main():
                         "other ranks' messages replayed from a recording of the full world" % (
                             args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk, rank),
             "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk, "measured_rank": rank,
-            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "kernel"),
+            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged"),
             "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64")),
         },
         "parity_bit_exact": parity,
@@ -346,7 +347,7 @@ def main():
                 "device_GBps": round(world_bytes / world_sec * 1e-9, 1),
                 "frac_of_hbm_peak": round(world_bytes / world_sec * 1e-9 / HBM_PEAK_GBPS, 4),
             },
-            "rank_zero_copy_landing": direct,
+            "rank_with_copy_kernel_landing": copied,
             "streams_per_rank": st[0]["streams_created"],
             "issue": "eager" if args.no_graph else "hip graph replay",
             "graph_calls_eager_captured_replayed": list(graph_counters),

@@ -34,7 +34,7 @@ def check(algo, bufs, chunk=None, **kw):
     return rep
 
 
-@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
 @pytest.mark.parametrize("fuse", [1, 3, 48])
 @pytest.mark.parametrize("world", [2, 3, 4, 5, 8])
 def test_ring_matches_oracle(world, fuse, landing):
@@ -44,7 +44,7 @@ def test_ring_matches_oracle(world, fuse, landing):
         check(RING, rand_bufs(world, n, seed=n), chunk, max_fuse=fuse, landing=landing, seed=world * 7 + fuse)
 
 
-@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
 @pytest.mark.parametrize("fuse", [1, 3, 48])
 @pytest.mark.parametrize("world", [2, 4, 8, 16])
 def test_rabenseifner_matches_oracle(world, fuse, landing):
@@ -58,7 +58,7 @@ def test_rabenseifner_matches_oracle(world, fuse, landing):
 def test_many_random_schedules(algo, world):
     bufs = rand_bufs(world, 777, seed=42)
     for seed in range(12):
-        check(algo, bufs, 32, max_fuse=1 + seed % 5, landing=seed % 3, seed=seed, streams=1 + seed % 4)
+        check(algo, bufs, 32, max_fuse=1 + seed % 5, landing=seed % 4, seed=seed, streams=1 + seed % 4)
 
 
 @pytest.mark.parametrize("algo,world", [(RING, 4), (RABEN, 4)])
@@ -78,7 +78,7 @@ def test_tiny_pool_forces_slot_reuse(algo, world):
 def test_threads_one_per_rank(algo, world):
     bufs = rand_bufs(world, 3000, seed=8)
     for rep_i in range(3):
-        check(algo, bufs, 64, max_fuse=4, landing=rep_i % 3, threaded=True, seed=rep_i)
+        check(algo, bufs, 64, max_fuse=4, landing=1 + rep_i % 3, threaded=True, seed=rep_i)
 
 
 @pytest.mark.parametrize("algo", [RING, RABEN])
@@ -87,13 +87,14 @@ def test_repeated_calls_reuse_events_and_slots(algo):
     rep = check(algo, bufs, 64, max_fuse=3, repeats=4, seed=1)
     assert rep.rank0.calls == 4
     check(algo, bufs, 64, max_fuse=3, repeats=3, threaded=True, seed=2)
+    check(algo, bufs, 64, max_fuse=3, repeats=4, landing=3, seed=3)  # staging slots are recycled across calls
 
 
 @pytest.mark.parametrize("algo,world", [(RING, 3), (RING, 4), (RABEN, 4)])
 def test_in_place(algo, world):
     bufs = rand_bufs(world, 1500, seed=6)
     orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs)
-    for landing in (0, 1, 2):
+    for landing in (0, 1, 2, 3):
         rc, recv, rep = S.allreduce(algo, bufs, max_fuse=5, landing=landing, in_place=True, seed=landing)
         assert rc == 0, rep.error.decode()
         for r in range(world):
@@ -153,7 +154,7 @@ def test_work_per_rank_matches_the_schedule():
     assert rep.rank0.reduce_segments == 3 * q and rep.rank0.gather_bytes == 3 * q * chunk
 
 
-@pytest.mark.parametrize("landing", [0, 1, 2])
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
 @pytest.mark.parametrize("algo,world", [(RING, 2), (RING, 4), (RING, 5), (RABEN, 4), (RABEN, 8)])
 def test_one_rank_replayed_against_recorded_peers(algo, world, landing):
     # a rank run alone against the recording of its incoming traffic must end with the very result
@@ -305,7 +306,7 @@ def test_randomised_shapes_and_knobs():
         if chunk is not None and dtype == np.float64:
             chunk *= 2
         bufs = [(np.random.default_rng(case * 100 + r).standard_normal(n) * 50).astype(dtype) for r in range(world)]
-        kw = dict(max_fuse=int(rng.integers(1, 65)), landing=int(rng.integers(0, 3)), seed=case,
+        kw = dict(max_fuse=int(rng.integers(1, 65)), landing=int(rng.integers(0, 4)), seed=case,
                   streams=int(rng.integers(1, 9)), pool_bytes=int(rng.choice([512, 4096, 65536])),
                   in_place=bool(rng.random() < 0.2), threaded=bool(rng.random() < 0.15))
         orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs, chunk)

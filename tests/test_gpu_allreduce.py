@@ -28,7 +28,7 @@ def kat_answer(world, n):
 
 # ------------------------------------------------------------------ engines vs oracle
 
-@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("fuse", [1, 4, 48])
 @pytest.mark.parametrize("world_size", [2, 3, 4, 8])
 def test_ring_matches_oracle(world_size, fuse, landing):
@@ -39,7 +39,7 @@ def test_ring_matches_oracle(world_size, fuse, landing):
             G.check_against_oracle(w, H.RING, rand_bufs(world_size, n, seed=n), chunk)
 
 
-@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("fuse", [1, 4, 48])
 @pytest.mark.parametrize("world_size", [2, 4, 8, 16])
 def test_rabenseifner_matches_oracle(world_size, fuse, landing):
@@ -89,7 +89,7 @@ def test_odd_chunk_offsets_keep_vector_path_correct():
         G.check_against_oracle(w, H.RING, rand_bufs(5, 1003))
 
 
-@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 4, None), (H.RING, 8, 4096), (H.RABENSEIFNER, 8, None)])
 def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
     # the single-thread driver records a call shape on its second use and replays it afterwards;
@@ -126,7 +126,7 @@ def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
         assert w.graph_counters()[0] == eager + 3
 
 
-@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT])
+@pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 8, 65536), (H.RING, 3, None), (H.RABENSEIFNER, 8, 65536)])
 def test_one_rank_replayed_against_recorded_peers(algo, world_size, chunk, landing):
     # the measured unit of the benchmark: one rank's complete schedule, peers replaced by a recording
