@@ -322,7 +322,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "BASELINE configs[%d]: %s allreduce, %d emulated ranks, %d fp32 (%.0f MiB) per rank, IBCOMM_CHUNKSIZE=%d; "
-                        "one step = rank %d's complete schedule on the GPU (its landings, reductions and gathers), the "
+                        "one step = rank %d's complete schedule on the GPU (its reductions and gathers, plus landing copies in the modes that make them), the "
                         "other ranks' messages replayed from a recording of the full world" % (
                             args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk, rank),
             "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk, "measured_rank": rank,

@@ -193,8 +193,8 @@ int ibcomm_hip_comm_set_max_fuse(ibcomm_hip_comm* comm, int max_chunks_per_launc
 /* How a message reaches the reduction: 0 = hipMemcpyAsync into a pool slot, 1 = one copy-kernel
  * launch for all messages of a pass, 2 = the reduction reads the sender's buffer directly, 3 = as 2,
  * and a partial sum that is only forwarded is produced into a pool slot (send staging) instead of
- * recvbuf, where the next rank's reduction reads it.  IBCOMM_HIP_LANDING = memcpy | kernel | direct |
- * staged sets the initial mode. */
+ * recvbuf, where the next rank's reduction reads it (the default).  IBCOMM_HIP_LANDING = memcpy |
+ * kernel | direct | staged sets the initial mode. */
 int ibcomm_hip_comm_set_landing(ibcomm_hip_comm* comm, int mode);
 
 /* Host-side pipeline trace in the reference's seven categories and .dat format
