@@ -159,16 +159,29 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     import numpy as np
     bufs = [np.random.default_rng(900 + r).standard_normal(n).astype(np.float32) for r in range(world)]
     algo = O.RING_CPU if algo_name == "ring" else O.RABEN_CPU
+    recv = [np.empty_like(b) for b in bufs]
     times = []
     for i in range(6):  # 1 warm-up + 5 timed
         t0 = time.perf_counter()
-        rc, recv, _ = O.allreduce(algo, bufs, chunk if algo_name == "ring" else None)
+        rc = O.allreduce_into(algo, bufs, recv, chunk if algo_name == "ring" else None)
         t1 = time.perf_counter()
         assert rc == 0
         if i:
             times.append(t1 - t0)
-        del recv
+    del recv
     t = min(times)
+    # The reference's own CPU-runnable case and timing protocol (examples/allreduce.cpp:28-29, 87-94, 107-118):
+    # 4 ranks x 4,194,304 integer-valued floats, default chunking, 3 warm-ups then one timed run.
+    n1 = 4 * 1024 * 1024
+    bufs1 = [np.random.default_rng(r).integers(-1000, 1001, n1).astype(np.float32) for r in range(4)]
+    recv1 = [np.empty_like(b) for b in bufs1]
+    for i in range(4):
+        t0 = time.perf_counter()
+        rc = O.allreduce_into(O.RING_CPU, bufs1, recv1, None)
+        t_cfg1 = time.perf_counter() - t0
+        assert rc == 0
+    exact = np.sum(np.stack(bufs1).astype(np.int64), axis=0)
+    cfg1_ok = all(bool(np.array_equal(r.astype(np.int64), exact)) for r in recv1)
     single_n = 64 * 1024 * 1024  # 256 MiB per operand: memory-bound on any host
     single = O.lib().orc_time_reduce_f32(single_n, 3)
     return {
@@ -181,6 +194,8 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
         "seconds": round(t, 3),
         "seconds_median": round(sorted(times)[len(times) // 2], 3),
         "single_core_reduce_loop_GBps": round(12.0 * single_n / single * 1e-9, 2),
+        "config1_ring_4x16MiB": {"seconds": round(t_cfg1, 4), "algbw_GBps": round(n1 * 4 / t_cfg1 * 1e-9, 3), "threads": 4,
+                                 "protocol": "3 warm-ups + 1 timed run", "equals_exact_integer_sum": cfg1_ok},
     }
 
 

@@ -117,6 +117,14 @@ def allreduce(algo, sendbufs, chunksize=None, pool_block_bytes=0):
     return rc, recv, st
 
 
+def allreduce_into(algo, sendbufs, recvbufs, chunksize=None, pool_block_bytes=0):
+    """Like allreduce() into caller-owned contiguous recvbufs, with nothing but the oracle call inside
+    (what a timing loop wants). -> rc"""
+    st = Stats()
+    return lib().orc_allreduce(algo, DTYPE_OF[sendbufs[0].dtype], len(sendbufs), _ptr_array(sendbufs), _ptr_array(recvbufs),
+                               sendbufs[0].size, _env(chunksize), pool_block_bytes, C.byref(st))
+
+
 def wire_log(world):
     """{(src, dst): [(offset, n), ...]} of the last allreduce() call."""
     out = {}
