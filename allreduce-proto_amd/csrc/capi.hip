@@ -2,6 +2,7 @@
 // include/ibcomm_hip.h.
 #include "ibcomm_hip.h"
 
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -59,6 +60,7 @@ struct ibcomm_hip_fabric {
     graphs.clear();
   }
   Fabric<HipBackend> fabric;
+  std::mutex mu;                 // guards live_comms and the graph cache against concurrent create / destroy
   int live_comms = 0;
   int graph_mode = 1;            // 0 = always issue eagerly, 1 = capture a call shape on its second use
   hipStream_t origin = nullptr;  // stream the graphs are captured from and replayed on
@@ -113,7 +115,10 @@ int ibcomm_hip_comm_create(ibcomm_hip_fabric* fabric, int world_size, ibcomm_hip
     delete c;
     return rc;
   }
-  fabric->live_comms++;
+  {
+    std::lock_guard<std::mutex> lock(fabric->mu);
+    fabric->live_comms++;
+  }
   *out = c;
   return kOk;
 }
@@ -122,9 +127,12 @@ int ibcomm_hip_comm_destroy(ibcomm_hip_comm* comm) {
   if (!comm) return kOk;
   comm->comm.Abort();
   if (comm->comm.trace().enabled()) comm->comm.DumpTrace();  // the reference dumps in its destructor (cpp:145-147)
-  comm->owner->DropGraphs();  // recorded graphs point into this communicator's pool
-  comm->owner->has_last_eager = false;
-  comm->owner->live_comms--;
+  {
+    std::lock_guard<std::mutex> lock(comm->owner->mu);
+    comm->owner->DropGraphs();  // recorded graphs point into this communicator's pool
+    comm->owner->has_last_eager = false;
+    comm->owner->live_comms--;
+  }
   delete comm;
   return kOk;
 }
@@ -406,6 +414,7 @@ int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, cons
                                const size_t* len, void* stream) {
   if (DTypeSize(dtype) == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
   if (n_segments < 0 || n_segments > kMaxSegments) return Fail(kInvalidArgument, "at most %d segments per launch", kMaxSegments);
+  if (n_segments && (!dst || !a || !b || !len)) return Fail(kInvalidArgument, "null segment table");
   SegmentBatch batch;
   batch.count = n_segments;
   for (int i = 0; i < n_segments; i++) {
@@ -418,7 +427,8 @@ int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, cons
 
 int ibcomm_hip_split_buffer(size_t len, size_t sizeof_element, int world_size, const char* env_chunksize, size_t* starts,
                             size_t* ends, int cap, int* n_ranges) {
-  if (!n_ranges || sizeof_element == 0 || world_size < 1) return Fail(kInvalidArgument, "bad argument");
+  if (!n_ranges || sizeof_element == 0 || world_size < 1 || cap < 0 || (cap > 0 && (!starts || !ends)))
+    return Fail(kInvalidArgument, "bad argument");
   std::vector<Range> ranges;
   *n_ranges = 0;
   IBCOMM_RETURN_IF_ERROR(SplitBuffer(len, sizeof_element, world_size, env_chunksize, &ranges));

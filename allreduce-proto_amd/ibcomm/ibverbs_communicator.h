@@ -40,9 +40,9 @@ class IBVerbsCommunicator {
 
   ~IBVerbsCommunicator() {
     if (!comm_) return;
-    ibcomm_hip_comm_destroy(comm_);
     Registry& reg = registry();
     std::lock_guard<std::mutex> lock(reg.mu);
+    ibcomm_hip_comm_destroy(comm_);
     World& w = reg.worlds[world_size_];
     if (--w.users == 0) {
       ibcomm_hip_fabric_destroy(w.fabric);
