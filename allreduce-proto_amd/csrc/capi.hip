@@ -357,10 +357,11 @@ int ibcomm_hip_world_record(ibcomm_hip_comm* const* comms, int world_size, int r
   IBCOMM_RETURN_IF_ERROR(CollectWorld(comms, world_size, &cs));
   ibcomm_hip_fabric* f = comms[0]->owner;
   size_t log_bytes = 0;
-  IBCOMM_RETURN_IF_ERROR(cs[rank]->RecordingBytes(algo, dtype, len, &log_bytes));
+  bool descending = false;
+  IBCOMM_RETURN_IF_ERROR(cs[rank]->RecordingBytes(algo, dtype, len, &log_bytes, &descending));
   f->DropGraphs();  // replay graphs point into the log, which is about to be rewritten (and may move)
   f->has_last_eager = false;
-  IBCOMM_RETURN_IF_ERROR(f->fabric.StartRecording(rank, log_bytes));
+  IBCOMM_RETURN_IF_ERROR(f->fabric.StartRecording(rank, log_bytes, descending));
   f->eager_calls++;
   const int rc = RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, true);
   f->fabric.StopRecording();

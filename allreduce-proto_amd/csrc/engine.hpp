@@ -80,6 +80,9 @@ struct EngineStats {
   uint64_t pool_blocks = 0;
   uint64_t pool_bytes = 0;
   uint64_t progress_passes = 0;
+  uint64_t reduce_kernel_segments = 0;  // segments the reduction launches carried after merging contiguous chunks
+  uint64_t largest_reduce_elements = 0;  // the reduction launch with the most elements: its elements ...
+  uint64_t largest_reduce_kernel_segments = 0;  // ... and its kernel segments
 };
 
 template <class B>
@@ -206,7 +209,15 @@ class Communicator {
     posted_.assign(world_size_, std::deque<PostedSend>());
     pending_reduce_.clear();
     pending_gather_.clear();
-    IBCOMM_RETURN_IF_ERROR(pool_.GetController(plan_.part.ranges[0].size() * es_, &controller_));
+    // A slot needs spare bytes only if some chunk of recvbuf starts off a 16-byte boundary.  Without
+    // them, slots of a chunk size that is a multiple of 256 bytes lie back to back, so chunks that are
+    // neighbours in the buffers are neighbours in the pool too and merge into one kernel segment.
+    const size_t chunk_bytes = plan_.part.ranges[0].size() * es_;
+    const bool phase_margin = (reinterpret_cast<uintptr_t>(recvbuf_) & 15) != 0 || (chunk_bytes & 15) != 0;
+    // The ring's queues visit the chunks of a group from the last to the first, the halving windows
+    // from the first to the last; the pool hands out its slots in the same direction.
+    IBCOMM_RETURN_IF_ERROR(pool_.GetController(chunk_bytes, phase_margin, Descending(plan_), &controller_));
+    reduce_runs_ = gather_runs_ = 0;
     active_ = true;
     return kOk;
   }
@@ -290,8 +301,9 @@ class Communicator {
     return Finish(true);
   }
 
-  // Bytes of log a recording of this rank's side of the given collective needs.
-  int RecordingBytes(int algo, int dtype, size_t len_elements, size_t* out) {
+  // Bytes of log a recording of this rank's side of the given collective needs, and whether that
+  // collective visits neighbouring chunks downwards.
+  int RecordingBytes(int algo, int dtype, size_t len_elements, size_t* out, bool* descending = nullptr) {
     Plan p;
     const size_t es = DTypeSize(dtype);
     if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
@@ -299,6 +311,7 @@ class Communicator {
     size_t total = 0;
     for (const RecvOp& r : p.recvs) total += (p.part.ranges[r.chunk].size() * es + 255) & ~size_t(255);
     *out = total;
+    if (descending) *descending = Descending(p);
     return kOk;
   }
 
@@ -376,7 +389,10 @@ class Communicator {
   struct PendingRecv {
     int op = 0;              // index into plan_.recvs
     Message msg;
-    Memory<B>* slot = nullptr;  // landing slot; null for gathers and in direct mode
+    Memory<B>* slot = nullptr;   // landing slot; null for gathers and when the message is read in place
+    Memory<B>* stage = nullptr;  // send-staging slot the result goes to; null when it goes to recvbuf
+    int joins = 0;               // +1 / -1: its operands continue those of the pending entry before it,
+                                 // upwards / downwards in memory, so both share a kernel segment; 0: new segment
   };
   struct PostedSend {
     uint64_t ticket;
@@ -388,12 +404,67 @@ class Communicator {
     bool active = false;
   };
 
+  static bool Descending(const Plan& p) { return p.recvs.size() > 1 && p.recvs[1].chunk < p.recvs[0].chunk; }
+
   bool ZeroCopyReceive() const { return landing_ == kLandDirect || landing_ == kLandStaged; }
 
   char* RecvPtr(int chunk) const { return recvbuf_ + plan_.part.ranges[chunk].begin * es_; }
   const char* SendPtr(int chunk) const { return sendbuf_ + plan_.part.ranges[chunk].begin * es_; }
   size_t ChunkElems(int chunk) const { return plan_.part.ranges[chunk].size(); }
   size_t ChunkBytes(int chunk) const { return plan_.part.ranges[chunk].size() * es_; }
+
+  // The three pointers of the reduction of one pending partial sum.
+  const void* IncomingOf(const PendingRecv& p) const {
+    return ZeroCopyReceive() ? p.msg.src : p.slot->LandingFor(RecvPtr(plan_.recvs[p.op].chunk));
+  }
+  const void* OwnOf(const PendingRecv& p) const {
+    const RecvOp& r = plan_.recvs[p.op];
+    return r.kind == kReduceWithSendbuf ? SendPtr(r.chunk) : static_cast<const char*>(RecvPtr(r.chunk));
+  }
+  void* ResultOf(const PendingRecv& p) const {
+    const int c = plan_.recvs[p.op].chunk;
+    return p.stage ? p.stage->LandingFor(RecvPtr(c)) : RecvPtr(c);
+  }
+  // +1 if `next` starts where `prev` ends, -1 if it ends where `prev` starts, else 0.
+  static int Adjacent(const void* prev, size_t prev_bytes, const void* next, size_t next_bytes) {
+    const char* p = static_cast<const char*>(prev);
+    const char* n = static_cast<const char*>(next);
+    if (p + prev_bytes == n) return 1;
+    if (n + next_bytes == p) return -1;
+    return 0;
+  }
+  // Does the reduction of `next` continue the reduction of `prev` in all three operands, in the
+  // direction `run` the segment has grown in so far (0 = either)?  Returns the direction or 0.
+  int ReduceJoins(const PendingRecv& prev, const PendingRecv& next, int run) const {
+    const size_t pb = ChunkBytes(plan_.recvs[prev.op].chunk), nb = ChunkBytes(plan_.recvs[next.op].chunk);
+    const int d = Adjacent(ResultOf(prev), pb, ResultOf(next), nb);
+    if (d == 0 || (run != 0 && d != run)) return 0;
+    if (Adjacent(IncomingOf(prev), pb, IncomingOf(next), nb) != d || Adjacent(OwnOf(prev), pb, OwnOf(next), nb) != d) return 0;
+    return d;
+  }
+  int GatherJoins(const PendingRecv& prev, const PendingRecv& next, int run) const {
+    const int pc = plan_.recvs[prev.op].chunk, nc = plan_.recvs[next.op].chunk;
+    const int d = Adjacent(RecvPtr(pc), ChunkBytes(pc), RecvPtr(nc), ChunkBytes(nc));
+    if (d == 0 || (run != 0 && d != run)) return 0;
+    return Adjacent(prev.msg.src, ChunkBytes(pc), next.msg.src, ChunkBytes(nc)) == d ? d : 0;
+  }
+  // Adds a segment to a launch: a new entry, or (joins = +1 / -1) grown onto the end / the front of the last one.
+  static void AppendSegment(SegmentBatch* batch, const Segment& seg, int joins) {
+    if (joins == 0 || batch->count == 0) {
+      batch->seg[batch->count++] = seg;
+      return;
+    }
+    Segment& last = batch->seg[batch->count - 1];
+    if (joins < 0) {
+      last.dst = seg.dst;
+      last.a = seg.a;
+      last.b = seg.b;
+    }
+    last.n += seg.n;
+  }
+  // Chunks one launch may carry: the knob, or any number when the knob is at its ceiling (then only
+  // the number of kernel segments, after merging, bounds a launch).
+  size_t ChunkLimit() const { return max_fuse_ >= kMaxSegments ? SIZE_MAX : static_cast<size_t>(max_fuse_); }
 
   void ReleaseCall() {
     stats_.slots_high_water = std::max<uint64_t>(stats_.slots_high_water, controller_.high_water());
@@ -510,8 +581,11 @@ class Communicator {
       // messages at the same time.
       if (r.kind == kGather) {
         IBCOMM_RETURN_IF_ERROR(FlushReduces());
+        if (!pending_gather_.empty()) p.joins = GatherJoins(pending_gather_.back(), p, pending_gather_.back().joins);
+        if (p.joins == 0 && gather_runs_ == kMaxSegments) IBCOMM_RETURN_IF_ERROR(FlushGathers());
+        if (p.joins == 0) gather_runs_++;
         pending_gather_.push_back(p);
-        if (static_cast<int>(pending_gather_.size()) >= max_fuse_) IBCOMM_RETURN_IF_ERROR(FlushGathers());
+        if (pending_gather_.size() >= ChunkLimit()) IBCOMM_RETURN_IF_ERROR(FlushGathers());
       } else {
         IBCOMM_RETURN_IF_ERROR(FlushGathers());
         // Segments of one launch run concurrently: a chunk whose previous partial sum is still
@@ -522,9 +596,15 @@ class Communicator {
           TraceScope scope(&trace_, Trace::kIssueRecv);
           if (!ZeroCopyReceive()) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
         }
+        // Nobody on this rank reads a partial sum that is only forwarded: it is produced where the
+        // next rank will fetch it.
+        if (landing_ == kLandStaged && plan_.forward_only[p.op] >= 0) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.stage));
+        if (!pending_reduce_.empty()) p.joins = ReduceJoins(pending_reduce_.back(), p, pending_reduce_.back().joins);
+        if (p.joins == 0 && reduce_runs_ == kMaxSegments) IBCOMM_RETURN_IF_ERROR(FlushReduces());
+        if (p.joins == 0) reduce_runs_++;
         chunk_in_batch_[r.chunk] = 1;
         pending_reduce_.push_back(p);
-        if (static_cast<int>(pending_reduce_.size()) >= max_fuse_) IBCOMM_RETURN_IF_ERROR(FlushReduces());
+        if (pending_reduce_.size() >= ChunkLimit()) IBCOMM_RETURN_IF_ERROR(FlushReduces());
       }
       next_recv_++;
       stats_.messages_received++;
@@ -548,7 +628,7 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
         IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
-        batch.seg[batch.count++] = Segment{RecvPtr(c), nullptr, p.msg.src, nullptr, ChunkElems(c)};
+        AppendSegment(&batch, Segment{RecvPtr(c), nullptr, p.msg.src, nullptr, ChunkElems(c)}, p.joins);
         stats_.gather_bytes += ChunkBytes(c);
       }
       IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 2));
@@ -582,6 +662,7 @@ class Communicator {
       }
     }
     pending_gather_.clear();
+    gather_runs_ = 0;
     return kOk;
   }
 
@@ -623,7 +704,19 @@ class Communicator {
           PendingRecv& p = pending_reduce_[i];
           const int c = plan_.recvs[p.op].chunk;
           IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.slot));
-          copy.seg[copy.count++] = Segment{p.slot->LandingFor(RecvPtr(c)), nullptr, p.msg.src, nullptr, ChunkElems(c)};
+          // the slots of a run continue one another; the sources may or may not
+          int joins = 0;
+          if (p.joins != 0 && copy.count > 0) {
+            const PendingRecv& q = pending_reduce_[i - 1];
+            const int qc = plan_.recvs[q.op].chunk;
+            if (Adjacent(q.msg.src, ChunkBytes(qc), p.msg.src, ChunkBytes(c)) == p.joins) joins = p.joins;
+          }
+          if (joins == 0 && copy.count == kMaxSegments) {
+            IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
+            stats_.landing_copies++;
+            copy.count = 0;
+          }
+          AppendSegment(&copy, Segment{p.slot->LandingFor(RecvPtr(c)), nullptr, p.msg.src, nullptr, ChunkElems(c)}, joins);
           stats_.landing_bytes += ChunkBytes(c);
         }
         IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
@@ -645,29 +738,24 @@ class Communicator {
       const PendingRecv& p = pending_reduce_[i];
       const RecvOp& r = plan_.recvs[p.op];
       const int c = r.chunk;
-      const void* incoming = ZeroCopyReceive() ? p.msg.src : p.slot->LandingFor(RecvPtr(c));
-      const void* own;
-      if (r.kind == kReduceWithSendbuf) {
-        own = SendPtr(c);
-      } else {
-        own = RecvPtr(c);
-        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));  // the previous halving step's sum
+      if (r.kind != kReduceWithSendbuf) IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));  // the previous halving step's sum
+      if (p.stage) {
+        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.stage));
+        staged_[p.op] = p.stage;
       }
-      void* result = RecvPtr(c);
-      if (landing_ == kLandStaged && plan_.forward_only[p.op] >= 0) {
-        // Nobody on this rank reads this partial sum: produce it where the next rank will fetch it.
-        Memory<B>* stage = nullptr;
-        IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&stage));
-        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, stage));
-        staged_[p.op] = stage;
-        result = stage->LandingFor(RecvPtr(c));
-      }
-      batch.seg[batch.count++] = Segment{result, nullptr, incoming, own, ChunkElems(c)};
+      AppendSegment(&batch, Segment{ResultOf(p), nullptr, IncomingOf(p), OwnOf(p), ChunkElems(c)}, p.joins);
       stats_.reduce_elements += ChunkElems(c);
     }
     IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 0));
     stats_.reduce_launches++;
     stats_.reduce_segments += n;
+    stats_.reduce_kernel_segments += batch.count;
+    uint64_t launch_elements = 0;
+    for (int i = 0; i < batch.count; i++) launch_elements += batch.seg[i].n;
+    if (launch_elements > stats_.largest_reduce_elements) {
+      stats_.largest_reduce_elements = launch_elements;
+      stats_.largest_reduce_kernel_segments = batch.count;
+    }
     OpState done;
     IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
     trace_.Mark(Trace::kIssueReduKernel);
@@ -682,6 +770,7 @@ class Communicator {
       chunk_in_batch_[r.chunk] = 0;
     }
     pending_reduce_.clear();
+    reduce_runs_ = 0;
     return kOk;
   }
 
@@ -750,6 +839,7 @@ class Communicator {
   std::vector<char> chunk_in_batch_;      // per chunk: a reduction of it sits in pending_reduce_
   std::vector<std::deque<PostedSend>> posted_;  // per peer: sends awaiting completion, oldest first
   std::vector<PendingRecv> pending_reduce_, pending_gather_;
+  int reduce_runs_ = 0, gather_runs_ = 0;  // kernel segments the pending lists will merge into
   std::vector<Event> pull_events_;
   std::vector<Event> events_[2];
   int arena_ = 0;

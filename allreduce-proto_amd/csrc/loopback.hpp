@@ -100,9 +100,13 @@ class Fabric {
       e.from = from;
       e.bytes = out->bytes;
       e.gate = sends_posted;
-      e.offset = log_used_;
-      log_used_ += (out->bytes + 255) & ~size_t(255);
-      out->record_to = log_used_ <= log_bytes_ ? log_base_ + e.offset : nullptr;
+      const size_t rounded = (out->bytes + 255) & ~size_t(255);
+      const bool fits = log_used_ + rounded <= log_need_;
+      // The log is filled in the direction the chunks are visited in, so that payloads of chunks
+      // that are neighbours in the buffers are neighbours in the log, as they are in the pool.
+      e.offset = !fits ? 0 : (log_descending_ ? log_need_ - log_used_ - rounded : log_used_);
+      log_used_ += rounded;
+      out->record_to = fits ? log_base_ + e.offset : nullptr;
       log_.push_back(e);
     }
     return true;
@@ -179,8 +183,9 @@ class Fabric {
   // dependency on upstream ranks does), and its own sends complete immediately.
 
   // Arms recording for the next collective.  log_bytes must cover the payload of every message
-  // `rank` will take (each rounded up to 256 bytes).
-  int StartRecording(int rank, size_t log_bytes) {
+  // `rank` will take (each rounded up to 256 bytes); `descending` says that the collective visits
+  // neighbouring chunks from the higher address to the lower.
+  int StartRecording(int rank, size_t log_bytes, bool descending = false) {
     StopReplay();
     if (log_base_ && log_bytes_ < log_bytes) {
       B::Free(log_base_);
@@ -195,13 +200,15 @@ class Fabric {
     }
     log_.clear();
     log_used_ = 0;
+    log_need_ = log_bytes;
+    log_descending_ = descending;
     record_rank_ = rank;
     recorded_rank_ = -1;
     return 0;
   }
   // Ends recording; the log now describes `rank`'s side of the collective just run.
   void StopRecording() {
-    if (record_rank_ >= 0 && log_used_ <= log_bytes_) recorded_rank_ = record_rank_;
+    if (record_rank_ >= 0 && log_used_ <= log_need_) recorded_rank_ = record_rank_;
     record_rank_ = -1;
   }
   int recording_rank() const { return record_rank_; }
@@ -276,7 +283,8 @@ class Fabric {
   int recorded_rank_ = -1;  // rank the finished log belongs to
   int replay_rank_ = -1;    // rank currently running against the log
   char* log_base_ = nullptr;
-  size_t log_bytes_ = 0, log_used_ = 0, log_cursor_ = 0;
+  size_t log_bytes_ = 0, log_need_ = 0, log_used_ = 0, log_cursor_ = 0;
+  bool log_descending_ = false;
   std::vector<LogEntry> log_;
 };
 

@@ -87,6 +87,7 @@ class MemoryController {
 
   MemoryPool<B>* pool_ = nullptr;
   size_t stride_ = 0;
+  bool descending_ = false;
   std::vector<std::unique_ptr<Memory<B>>> slots_;
   std::deque<Memory<B>*> vacant_;
   int held_ = 0;
@@ -119,12 +120,16 @@ class MemoryPool {
   }
 
   // One controller at a time (memory_pool.h:111-121).
-  int GetController(size_t chunk_bytes, MemoryController<B>* c) {
+  // With phase_margin every slot keeps 16 spare bytes (see Memory::LandingFor); without, slots of a
+  // chunk size that is a multiple of 256 bytes are contiguous.  Slots are first handed out from the
+  // lowest address upwards, or with `descending` from the highest downwards.
+  int GetController(size_t chunk_bytes, bool phase_margin, bool descending, MemoryController<B>* c) {
     if (controller_in_use_) return Fail(kNotSupported, "Currently, MemoryController is in use.");
     if (chunk_bytes == 0) return Fail(kInvalidArgument, "chunk size must be positive");
     controller_in_use_ = true;
     c->pool_ = this;
-    c->stride_ = (chunk_bytes + 16 + 255) & ~size_t(255);
+    c->stride_ = (chunk_bytes + (phase_margin ? 16 : 0) + 255) & ~size_t(255);
+    c->descending_ = descending;
     c->slots_.clear();
     c->vacant_.clear();
     c->held_ = 0;
@@ -226,7 +231,10 @@ void MemoryController<B>::Carve(char* block, size_t block_bytes) {
   // Slots are reused first-in first-out and a pass holds at most one launch's worth of them, so
   // beyond a few hundred more slots buy nothing; tiny chunks would otherwise yield millions.
   constexpr size_t kMaxSlotsPerBlock = 1024;
-  for (size_t i = 0; (i + 1) * stride_ <= block_bytes && i < kMaxSlotsPerBlock; i++) {
+  size_t count = block_bytes / stride_;
+  if (count > kMaxSlotsPerBlock) count = kMaxSlotsPerBlock;
+  for (size_t k = 0; k < count; k++) {
+    const size_t i = descending_ ? count - 1 - k : k;
     slots_.emplace_back(new Memory<B>());
     Memory<B>* m = slots_.back().get();
     m->base = block + i * stride_;

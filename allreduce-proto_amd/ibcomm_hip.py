@@ -37,7 +37,8 @@ class Stats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "calls", "reduce_launches", "reduce_segments", "reduce_elements", "landing_copies", "landing_bytes",
         "gather_copies", "gather_bytes", "messages_sent", "messages_received", "events_recorded", "stream_waits",
-        "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes")]
+        "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes", "reduce_kernel_segments",
+        "largest_reduce_elements", "largest_reduce_kernel_segments")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

@@ -238,27 +238,6 @@ def main():
     sp = [t.data_ptr() for t in send]
     rp = [t.data_ptr() for t in recv]
 
-    # Shape of the dominant reduction launch of rank 0, from its plan: one ring step reduces one chunk
-    # group; the first Rabenseifner halving step reduces half of all groups (the largest window).
-    p = H.Plan(algo, world, 0, n, 4, chunk)
-    fuse = args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64"))
-    if algo == H.RING:
-        per_step = len(p.ranges) // world
-    else:
-        per_step = sum(1 for _, peer, kind in p.recvs if kind == 0)
-    leg_segments = max(1, min(fuse, per_step))
-    seg_elems = p.ranges[0][1] - p.ranges[0][0]
-
-    if args.only_roofline:
-        # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
-        # counters collected over this command can be calibrated against a known traffic
-        for _ in range(3):
-            recv[0].copy_(send[0])
-        torch.cuda.synchronize()
-        print(json.dumps({"only_roofline": True, "config": args.config,
-                          "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)}))
-        return
-
     def timed(call, steps, warm):
         for _ in range(warm):
             assert call() == 0, H.last_error()
@@ -292,6 +271,21 @@ def main():
         w.reset_stats()
         assert w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n) == 0, H.last_error()
         st_rank = w.stats(rank)
+        # Shape of the dominant reduction launch of the rank, as the engine issued it: one ring step
+        # reduces one chunk group, the first Rabenseifner halving step half of all groups; chunks that
+        # follow one another in all three operands share a kernel segment.
+        leg_segments = max(1, st_rank["largest_reduce_kernel_segments"])
+        seg_elems = st_rank["largest_reduce_elements"] // leg_segments
+
+        if args.only_roofline:
+            # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
+            # counters collected over this command can be calibrated against a known traffic
+            for _ in range(3):
+                recv[0].copy_(send[0])
+            torch.cuda.synchronize()
+            print(json.dumps({"only_roofline": True, "config": args.config,
+                              "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)}))
+            return
         sec_per_step = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
         parity = parity and bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
         del out
@@ -318,7 +312,8 @@ def main():
 
     rank_bytes = device_bytes(st_rank)
     world_bytes = sum(device_bytes(s) for s in st)
-    segs_per_launch = round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"]), 2)
+    chunks_per_launch = round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"]), 2)
+    segs_per_launch = round(st_rank["reduce_kernel_segments"] / max(1, st_rank["reduce_launches"]), 2)
 
     algbw = n * 4 / sec_per_step * 1e-9
     world_algbw = n * 4 / world_sec * 1e-9
@@ -351,7 +346,8 @@ def main():
             "rank_device_GBps": round(rank_bytes / sec_per_step * 1e-9, 1),
             "rank_frac_of_hbm_peak": round(rank_bytes / sec_per_step * 1e-9 / HBM_PEAK_GBPS, 4),
             "rank_reduce_launches_per_step": st_rank["reduce_launches"],
-            "rank_mean_segments_per_launch": segs_per_launch,
+            "rank_mean_chunks_per_launch": chunks_per_launch,
+            "rank_mean_kernel_segments_per_launch": segs_per_launch,
             "rank_reduce_elements_per_step": st_rank["reduce_elements"],
             "rank_landing_launches_per_step": st_rank["landing_copies"],
             "rank_gather_launches_per_step": st_rank["gather_copies"],

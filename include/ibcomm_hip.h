@@ -188,7 +188,9 @@ int ibcomm_hip_plan_send(const ibcomm_hip_plan* plan, int k, int* chunk, int* pe
 
 /* ---- knobs and counters --------------------------------------------------------------------- */
 
-/* Chunks reduced per kernel launch at most (1 = one launch per chunk, like the reference). */
+/* Chunks reduced per kernel launch at most (1 = one launch per chunk, like the reference).  At its
+ * ceiling and default, ibcomm_hip_max_segments(), a launch takes every chunk that is ready, however
+ * many, as long as they merge into that many kernel segments. */
 int ibcomm_hip_comm_set_max_fuse(ibcomm_hip_comm* comm, int max_chunks_per_launch);
 /* How a message reaches the reduction: 0 = hipMemcpyAsync into a pool slot, 1 = one copy-kernel
  * launch for all messages of a pass, 2 = the reduction reads the sender's buffer directly, 3 = as 2,
@@ -210,7 +212,7 @@ int ibcomm_hip_comm_dump_trace(ibcomm_hip_comm* comm);
 typedef struct {
   uint64_t calls;
   uint64_t reduce_launches;
-  uint64_t reduce_segments;
+  uint64_t reduce_segments;        /* chunks reduced */
   uint64_t reduce_elements;
   uint64_t landing_copies;
   uint64_t landing_bytes;
@@ -226,6 +228,10 @@ typedef struct {
   uint64_t pool_blocks;
   uint64_t pool_bytes;
   uint64_t progress_passes;
+  uint64_t reduce_kernel_segments; /* kernel segments of the reduction launches: chunks that follow one
+                                      another in all three operands are merged into one segment */
+  uint64_t largest_reduce_elements;        /* the reduction launch with the most elements: its elements */
+  uint64_t largest_reduce_kernel_segments; /* ... and its kernel segments */
 } ibcomm_hip_stats;
 
 int ibcomm_hip_comm_stats(ibcomm_hip_comm* comm, ibcomm_hip_stats* out);

@@ -18,7 +18,8 @@ class EngineStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "calls", "reduce_launches", "reduce_segments", "reduce_elements", "landing_copies", "landing_bytes",
         "gather_copies", "gather_bytes", "messages_sent", "messages_received", "events_recorded", "stream_waits",
-        "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes")]
+        "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes", "reduce_kernel_segments",
+        "largest_reduce_elements", "largest_reduce_kernel_segments")]
 
 
 class Report(C.Structure):
@@ -46,10 +47,11 @@ DT = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.float64): 2, n
 
 
 def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, threaded=False, repeats=1,
-              pool_bytes=1 << 16, in_place=False, streams=None):
+              pool_bytes=1 << 16, in_place=False, streams=None, copy=True):
     """-> (rc, [recvbuf per rank], Report).  Environment knobs are set for the duration of the call."""
     world = len(sendbufs)
-    sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]
+    if copy:  # copy=False: run on the caller's arrays, whatever their alignment
+        sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]
     n = sendbufs[0].size
     if in_place:
         recv = sendbufs

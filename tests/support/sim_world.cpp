@@ -261,12 +261,12 @@ int sim_pool_rules(int* second_controller, unsigned long long* block_bytes, int*
   *block_bytes = c.pool().block_bytes();
   *max_streams = c.pool().max_streams();
   MemoryController<SimBackend> a, b;
-  int rc2 = c.pool().GetController(chunk_bytes, &a);
+  int rc2 = c.pool().GetController(chunk_bytes, true, false, &a);
   if (rc2 != kOk) return rc2;
   *slots_for_chunk = static_cast<int>(a.slot_count());
-  *second_controller = c.pool().GetController(chunk_bytes, &b);
+  *second_controller = c.pool().GetController(chunk_bytes, true, false, &b);
   a.Release();
-  rc2 = c.pool().GetController(chunk_bytes, &b);  // free again after release
+  rc2 = c.pool().GetController(chunk_bytes, true, false, &b);  // free again after release
   b.Release();
   return rc2;
 }
@@ -290,8 +290,9 @@ int sim_record_replay(int algo, int dtype, int world, const void* const* sendbuf
     raw.push_back(comms.back().get());
   }
   size_t log_bytes = 0;
-  if (rc == kOk) rc = raw[rank]->RecordingBytes(algo, dtype, len, &log_bytes);
-  if (rc == kOk) rc = fabric.StartRecording(rank, log_bytes);
+  bool descending = false;
+  if (rc == kOk) rc = raw[rank]->RecordingBytes(algo, dtype, len, &log_bytes, &descending);
+  if (rc == kOk) rc = fabric.StartRecording(rank, log_bytes, descending);
   if (rc == kOk) rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, true);
   fabric.StopRecording();
   raw[rank]->reset_stats();

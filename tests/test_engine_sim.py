@@ -35,7 +35,7 @@ def check(algo, bufs, chunk=None, **kw):
 
 
 @pytest.mark.parametrize("landing", [0, 1, 2, 3])
-@pytest.mark.parametrize("fuse", [1, 3, 48])
+@pytest.mark.parametrize("fuse", [1, 3, 48, 64])
 @pytest.mark.parametrize("world", [2, 3, 4, 5, 8])
 def test_ring_matches_oracle(world, fuse, landing):
     for n, chunk in [(world, None), (4 * world + 1, None), (1000 + world, None), (512, 16)]:
@@ -45,7 +45,7 @@ def test_ring_matches_oracle(world, fuse, landing):
 
 
 @pytest.mark.parametrize("landing", [0, 1, 2, 3])
-@pytest.mark.parametrize("fuse", [1, 3, 48])
+@pytest.mark.parametrize("fuse", [1, 3, 48, 64])
 @pytest.mark.parametrize("world", [2, 4, 8, 16])
 def test_rabenseifner_matches_oracle(world, fuse, landing):
     for n, chunk in [(world, None), (4 * world + 3, None), (2000 + world, None), (1024, 16)]:
@@ -152,6 +152,98 @@ def test_work_per_rank_matches_the_schedule():
     # Rabenseifner rank 0 of 4: halving windows of 2 and 1 groups
     rep = check(RABEN, bufs, chunk, max_fuse=1)
     assert rep.rank0.reduce_segments == 3 * q and rep.rank0.gather_bytes == 3 * q * chunk
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+def test_contiguous_chunks_merge_into_one_kernel_segment(landing):
+    # 256-byte chunks in 16-byte aligned buffers: pool slots lie back to back, so the 16 chunks of a
+    # ring step follow one another in every operand and each launch carries a single segment
+    world, n, chunk = 4, 4096, 256
+    bufs = rand_bufs(world, n, seed=5)
+    q = n * 4 // chunk // world
+    st = check(RING, bufs, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    assert st.reduce_segments == (world - 1) * q
+    assert st.reduce_launches == world - 1 and st.reduce_kernel_segments == world - 1
+    assert st.gather_copies == (world - 1 if landing else (world - 1) * q)
+    # Rabenseifner rank 0 of 4: two halving steps over 2 and 1 groups
+    st = check(RABEN, bufs, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    # (staged: the half of the first window that is passed on in the second step goes to send staging,
+    # the half that is kept goes to recvbuf, which makes two segments of the first launch)
+    assert st.reduce_launches == 2 and st.reduce_segments == 3 * q
+    assert st.reduce_kernel_segments == (3 if landing == 3 else 2)
+    # 64-byte chunks occupy 256-byte slots: nothing that passes through the pool can merge, while
+    # reductions that read and write the callers' buffers only (direct) still do
+    q = n * 4 // 64 // world
+    st = check(RING, bufs, 64, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    assert st.reduce_launches == world - 1
+    if landing == 2:
+        assert st.reduce_kernel_segments == world - 1
+    elif landing == 3:  # the last step writes recvbuf and reads the sender's slots
+        assert st.reduce_kernel_segments == (world - 1) * q
+    else:
+        assert st.reduce_kernel_segments == (world - 1) * q
+    # below the knob's ceiling the knob counts chunks, merged or not
+    st = check(RING, bufs, chunk, max_fuse=5, landing=landing, pool_bytes=1 << 20).rank0
+    assert st.reduce_launches == (world - 1) * 4  # 16 chunks per step, 5 at a time
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+def test_more_chunks_per_step_than_kernel_segments(landing):
+    # 130 chunks per ring step.  Merged they fit one launch; unmerged they need ceil(130 / 64) = 3.
+    world, q = 2, 130
+    bufs = rand_bufs(world, world * q * 64, seed=6)
+    st = check(RING, bufs, 256, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    assert st.reduce_segments == q and st.reduce_launches == 1 and st.reduce_kernel_segments == 1
+    # 64-byte chunks in 256-byte slots, three ranks (so that partial sums pass through send staging)
+    world = 3
+    bufs = rand_bufs(world, world * q * 16, seed=7)
+    st = check(RING, bufs, 64, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    assert st.reduce_segments == 2 * q
+    if landing == 2:
+        assert st.reduce_launches == 2 and st.reduce_kernel_segments == 2
+    else:
+        assert st.reduce_launches == 6 and st.reduce_kernel_segments == 2 * q
+    world = 2
+    # a pool of 40 slots is recycled several times within the step: slots come back out of address
+    # order, runs break where they do, and the result is the same
+    st = check(RING, rand_bufs(world, world * q * 64, seed=8), 256, max_fuse=64, landing=landing, pool_bytes=40 * 256).rank0
+    assert st.reduce_segments == q
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+@pytest.mark.parametrize("algo", [RING, RABEN])
+def test_replay_launches_the_merged_shapes_of_the_world(algo, landing):
+    # the recording log is laid out in the direction the chunks are visited in, so a rank replayed
+    # alone merges its chunks exactly as it does among real peers
+    world, n, chunk = 4, 4096, 256
+    bufs = rand_bufs(world, n, seed=11)
+    in_world = check(algo, bufs, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
+    rc, recv, out, rep = S.record_replay(algo, bufs, 0, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20)
+    assert rc == 0 and rep.races == 0, (rep.error, rep.first_race)
+    assert np.array_equal(O.bits(out), O.bits(recv[0]))
+    alone = rep.rank0
+    assert (alone.reduce_launches, alone.reduce_kernel_segments, alone.reduce_segments) == \
+        (in_world.reduce_launches, in_world.reduce_kernel_segments, in_world.reduce_segments)
+    assert alone.gather_copies == in_world.gather_copies
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+def test_recvbuf_off_the_16_byte_grid_keeps_the_phase_margin(landing):
+    # recvbuf starting 4 bytes past a 16-byte boundary: every slot keeps its spare bytes, landings
+    # share the phase of their target, nothing through the pool merges, results are unchanged
+    world, n = 4, 2048
+    bufs = rand_bufs(world, n, seed=9)
+    backing = [np.empty(n + 1, dtype=np.float32) for _ in range(world)]
+    sends = []
+    for b, src in zip(backing, bufs):
+        b[1:] = src
+        sends.append(b[1:])
+    assert all(s.ctypes.data % 16 == 4 for s in sends)
+    rc, recv, rep = S.allreduce(RING, sends, 256, max_fuse=64, landing=landing, in_place=True, pool_bytes=1 << 20, copy=False)
+    assert rc == 0 and rep.races == 0, (rep.error, rep.first_race)
+    _, want, _ = O.allreduce(O.RING_GPU, bufs, 256)
+    for r in range(world):
+        assert np.array_equal(O.bits(recv[r]), O.bits(want[r]))
 
 
 @pytest.mark.parametrize("landing", [0, 1, 2, 3])
