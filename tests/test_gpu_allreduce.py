@@ -29,7 +29,7 @@ def kat_answer(world, n):
 # ------------------------------------------------------------------ engines vs oracle
 
 @pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
-@pytest.mark.parametrize("fuse", [1, 4, 48])
+@pytest.mark.parametrize("fuse", [1, 4, 48, 64])
 @pytest.mark.parametrize("world_size", [2, 3, 4, 8])
 def test_ring_matches_oracle(world_size, fuse, landing):
     with H.World(world_size) as w:
@@ -40,7 +40,7 @@ def test_ring_matches_oracle(world_size, fuse, landing):
 
 
 @pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
-@pytest.mark.parametrize("fuse", [1, 4, 48])
+@pytest.mark.parametrize("fuse", [1, 4, 48, 64])
 @pytest.mark.parametrize("world_size", [2, 4, 8, 16])
 def test_rabenseifner_matches_oracle(world_size, fuse, landing):
     with H.World(world_size) as w:
@@ -355,6 +355,37 @@ def test_config_5_ring_32_ranks_2gib_ragged_tail():
         check_stripes_against_oracle(send, recv[0], H.RING, chunk, [0, 3, 4, 63, 124, 127])
         check_stripes_against_oracle(send, recv[31], H.RING, chunk, [127])
         del send, recv
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("algo,world_size", [(H.RING, 3), (H.RABENSEIFNER, 2)])
+def test_more_than_2_to_the_31_elements(algo, world_size):
+    # The reference indexes chunk ranges with int (ibverbs_communicator.cpp:676-677) and stops short of
+    # 2^31 elements; here offsets are size_t.  int32 data, so that the sum is exact in any order (wrapping).
+    n = 2**31 + 4099
+    free, _ = torch.cuda.mem_get_info()
+    if free < (2 * world_size * 4 * n) + 24 * 2**30:
+        pytest.skip("needs about %d GiB of free HBM" % ((2 * world_size * 4 * n >> 30) + 24))
+    with H.World(world_size) as w:
+        i = torch.arange(n, device="cuda", dtype=torch.int64)
+        send = [((i * 2654435761 + r * 40503) & 0xFFFFFFFF).to(torch.int32) for r in range(world_size)]
+        del i
+        recv = [torch.empty_like(t) for t in send]
+        ptrs = lambda ts: [t.data_ptr() for t in ts]  # noqa: E731
+        torch.cuda.synchronize()
+        assert w.allreduce_ptrs(algo, H.I32, ptrs(send), ptrs(recv), n) == 0, H.last_error()
+        torch.cuda.synchronize()
+        want = send[0].clone()
+        for t in send[1:]:
+            want += t
+        for r in range(world_size):
+            assert torch.equal(recv[r], want), "rank %d" % r
+        # the elements on either side of the 2^31 boundary and the ragged tail, on the host
+        for lo, hi in ((2**31 - 3, 2**31 + 3), (n - 5, n)):
+            host = sum(t[lo:hi].cpu().numpy().astype(np.int64) for t in send).astype(np.int32)
+            assert np.array_equal(recv[world_size - 1][lo:hi].cpu().numpy(), host)
+        assert w.stats(0)["reduce_elements"] > 2**30
+        del send, recv, want
     torch.cuda.empty_cache()
 
 
