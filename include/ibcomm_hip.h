@@ -92,8 +92,12 @@ int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const vo
  * the data is copied to the device, reduced by the device path above and copied back.  The sums and
  * their order are the same (ring: left fold from the owner of the chunk group under
  * SplitBuffer; Rabenseifner: balanced tree, which does not depend on how the buffer is cut), so the
- * results are bit-identical to the reference's.  One difference: the reference's CPU Rabenseifner does
- * not go through SplitBuffer and therefore accepts len_elements < world_size, which returns 4 here. */
+ * results are bit-identical to the reference's.  Two differences, both from the reference's CPU
+ * Rabenseifner cutting the buffer into world_size ranges of ceilDiv(len, world_size) elements instead
+ * of going through SplitBuffer (allreduce_cpu_impl.h:264-271): it accepts len_elements < world_size,
+ * which returns 4 here; and when (world_size - 1) * ceilDiv(len, world_size) > len (5 elements on 4
+ * ranks) one of its ranges is inverted and its size_t lengths wrap, whereas every
+ * len_elements >= world_size works here. */
 int ibcomm_hip_allreduce_ring_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,
                                    size_t len_elements);
 int ibcomm_hip_allreduce_rabenseifner_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf,

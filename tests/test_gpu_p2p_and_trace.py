@@ -98,3 +98,26 @@ def test_host_buffer_calls_match_the_reference_cpu_path(algo, oracle_algo, world
                 assert rcs == [0] * world_size, msgs
                 for r in range(world_size):
                     assert np.array_equal(O.bits(out[r]), O.bits(want[r])), "rank %d" % r
+
+
+@pytest.mark.parametrize("world_size,n", [(4, 5), (8, 13), (8, 1001), (4, 4)])
+def test_host_rabenseifner_lengths_the_reference_cannot_split(world_size, n):
+    # The reference's CPU Rabenseifner cuts the buffer into N ranges of ceilDiv(len, N) elements
+    # (allreduce_cpu_impl.h:264-271).  When (N-1) * ceilDiv(len, N) > len (5 elements on 4 ranks: ranges
+    # (0,2) (2,4) (4,5) (6,5)) a range is inverted and its size_t lengths wrap; the oracle refuses such
+    # input.  Here the host call goes through SplitBuffer like the device path, so every len >= N works,
+    # and the result is the balanced tree, which does not depend on how the buffer is cut.
+    import oracle_lib as O
+    host = [np.random.default_rng(70 + r).standard_normal(n).astype(np.float32) for r in range(world_size)]
+    if (-(-n // world_size)) * (world_size - 1) > n:
+        assert O.allreduce(O.RABEN_CPU, host)[0] == O.NOT_SUPPORTED
+    rc, want = O.closed_form_tree(host)
+    assert rc == 0
+    out = [np.full(n, 7.0, dtype=np.float32) for _ in range(world_size)]
+    with G.env(IBCOMM_CHUNKSIZE=None):
+        with H.World(world_size) as w:
+            rcs, msgs = w.allreduce_threads(H.RABENSEIFNER, H.F32, [h.ctypes.data for h in host], [o.ctypes.data for o in out], n, host=True)
+            assert rcs == [0] * world_size, msgs
+    for r in range(world_size):
+        assert np.array_equal(O.bits(out[r]), O.bits(want)), "rank %d" % r
+
