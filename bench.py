@@ -161,7 +161,7 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     algo = O.RING_CPU if algo_name == "ring" else O.RABEN_CPU
     recv = [np.empty_like(b) for b in bufs]
     times = []
-    for i in range(6):  # 1 warm-up + 5 timed
+    for i in range(16):  # 1 warm-up + 15 timed
         t0 = time.perf_counter()
         rc = O.allreduce_into(algo, bufs, recv, chunk if algo_name == "ring" else None)
         t1 = time.perf_counter()
@@ -189,7 +189,7 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
         "unit": "GB/s algbw",
         "cores": min(world, os.cpu_count() or 1),
         "kind": "port",
-        "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 5 after 1 warm-up, "
+        "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 15 after 1 warm-up, "
                   "one host thread per emulated rank on %d logical CPUs" % (algo_name, world, n, chunk, os.cpu_count() or 1),
         "seconds": round(t, 3),
         "seconds_median": round(sorted(times)[len(times) // 2], 3),
