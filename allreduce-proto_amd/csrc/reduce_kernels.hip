@@ -111,7 +111,50 @@ __global__ __launch_bounds__(THREADS) void SegmentKernel(const SegmentBatch batc
   }
 }
 
+// The common case on its own: every pointer of every segment on a 16-byte boundary, every length a
+// whole number of vectors, one destination, one vector per lane.  Without the peeling logic a
+// workgroup issues its loads a few hundred nanoseconds earlier, which a launch of a few tens of
+// megabytes feels (8192 short-lived workgroups over 256 CUs start in several rounds).
+template <typename T, typename V, int THREADS, int NT, bool ADD>
+__global__ __launch_bounds__(THREADS) void AlignedSegmentKernel(const SegmentBatch batch) {
+  const Segment s = batch.seg[blockIdx.y];
+  const uint64_t nvec = s.n / (16 / sizeof(T));
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * THREADS + threadIdx.x;
+  if (i >= nvec) return;
+  V v = LoadVec<(NT & 1) != 0>(static_cast<const V*>(s.a) + i);
+  if (ADD) v = v + LoadVec<(NT & 2) != 0>(static_cast<const V*>(s.b) + i);
+  StoreVec<(NT & 4) != 0>(static_cast<V*>(s.dst) + i, v);
+}
+
 namespace {
+
+int EnvInt(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
+
+template <typename T, typename V, int NT>
+hipError_t LaunchAlignedOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
+  if (batch.seg[0].b != nullptr)
+    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, 256, NT, true>), grid, dim3(256), 0, stream, batch);
+  else
+    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, 256, NT, false>), grid, dim3(256), 0, stream, batch);
+  return hipGetLastError();
+}
+
+template <typename T, typename V>
+hipError_t LaunchAligned(const SegmentBatch& batch, dim3 grid, int nt, hipStream_t stream) {
+  switch (nt & 7) {
+    case 0: return LaunchAlignedOne<T, V, 0>(batch, grid, stream);
+    case 1: return LaunchAlignedOne<T, V, 1>(batch, grid, stream);
+    case 2: return LaunchAlignedOne<T, V, 2>(batch, grid, stream);
+    case 3: return LaunchAlignedOne<T, V, 3>(batch, grid, stream);
+    case 4: return LaunchAlignedOne<T, V, 4>(batch, grid, stream);
+    case 5: return LaunchAlignedOne<T, V, 5>(batch, grid, stream);
+    case 6: return LaunchAlignedOne<T, V, 6>(batch, grid, stream);
+    default: return LaunchAlignedOne<T, V, 7>(batch, grid, stream);
+  }
+}
 
 template <typename T, typename V, int THREADS, int UNROLL, int NT>
 hipError_t LaunchOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
@@ -155,11 +198,6 @@ hipError_t LaunchThreads(const SegmentBatch& batch, dim3 grid, const LaunchTunin
   }
 }
 
-int EnvInt(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : fallback;
-}
-
 }  // namespace
 
 LaunchTuning DefaultTuning() {
@@ -181,15 +219,33 @@ hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuni
 
   uint64_t max_n = 0;
   const bool add = batch.seg[0].b != nullptr;
+  const uint64_t per_vec = 16 / es;
+  uintptr_t misfit = 0;  // any low pointer bit, any length remainder, any second destination
   for (int i = 0; i < batch.count; i++) {
     const Segment& s = batch.seg[i];
     if (s.n && (!s.dst || !s.a)) return hipErrorInvalidValue;
     if ((s.b != nullptr) != add) return hipErrorInvalidValue;  // a launch is all adds or all copies
     if (s.n > max_n) max_n = s.n;
+    if (s.n)
+      misfit |= ((reinterpret_cast<uintptr_t>(s.dst) | reinterpret_cast<uintptr_t>(s.a) | reinterpret_cast<uintptr_t>(s.b)) & 15) |
+                (s.n % per_vec) | reinterpret_cast<uintptr_t>(s.dst2);
   }
   if (max_n == 0) return hipSuccess;
 
-  const uint64_t per_vec = 16 / es;
+  static const bool fast_path_off = EnvInt("IBCOMM_HIP_NO_ALIGNED_KERNEL", 0) != 0;
+  if (misfit == 0 && tuning.threads == 256 && tuning.unroll == 1 && tuning.max_blocks_x == 0 && !fast_path_off) {
+    const uint64_t blocks = (max_n / per_vec + 255) / 256;
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
+    switch (dtype) {
+      case kF32: return LaunchAligned<float, f32x4>(batch, grid, tuning.nontemporal, stream);
+      case kI32: return LaunchAligned<uint32_t, u32x4>(batch, grid, tuning.nontemporal, stream);
+      case kF64: return LaunchAligned<double, f64x2>(batch, grid, tuning.nontemporal, stream);
+      case kI64: return LaunchAligned<uint64_t, u64x2>(batch, grid, tuning.nontemporal, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
+
   const uint64_t tile = static_cast<uint64_t>(tuning.threads) * tuning.unroll;
   uint64_t blocks = (max_n / per_vec + tile - 1) / tile;
   if (blocks == 0) blocks = 1;

@@ -17,6 +17,13 @@
 // segment whose three pointers share their 16-byte phase is peeled at head and
 // tail so the body stays vectorised even when a chunk starts at an odd element.
 //
+// Two kernels share that contract.  AlignedSegmentKernel takes the launches in which every pointer
+// is on a 16-byte boundary and every length a whole number of vectors (in practice all of the
+// engine's, since chunk sizes and buffers are aligned): load, add, store, nothing else, because
+// with one vector per lane a workgroup lives for one memory round trip and every instruction ahead
+// of its loads delays them.  SegmentKernel takes everything else (odd offsets, ragged tails, a
+// second destination, the tuning experiments).
+//
 // One IEEE-754 add per element, no multiply, so nothing can contract into an
 // FMA: results are bit-identical to the host's `float` add, provided fp32
 // denormals are kept (they are: the kernels are built without

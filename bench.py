@@ -146,7 +146,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
         "unit": "GB/s",
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get("%d segments x %d fp32" % (k, seg_elems)),
-        "kernel": "ibcomm_hip::SegmentKernel<float, float4, 256, 1, nontemporal, add>",
+        "kernel": "ibcomm_hip::AlignedSegmentKernel<float, float4, 256, nontemporal, add>",
         "launch_shape": "%d segments x %d fp32" % (k, seg_elems),
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
