@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the reduction kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
 # each calibrated against a device copy of known size; the summary with the commands is
 # profiles/segment_kernel_add_ring8_256MiB.md.  Shapes that have not been measured report null.
-MEASURED_TRAFFIC_BYTES = {"1 segments x 8388608 fp32": 100692365}
+MEASURED_TRAFFIC_BYTES = {"1 segments x 8388608 fp32": 100678989}
 
 CONFIGS = {
     # id: (algo name, ranks, elements per rank, IBCOMM_CHUNKSIZE, data)
