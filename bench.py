@@ -360,7 +360,7 @@ def main():
             },
             "rank_with_copy_kernel_landing": copied,
             "streams_per_rank": st[0]["streams_created"],
-            "issue": "eager" if args.no_graph else "hip graph replay",
+            "issue": "hip graph replay" if graph_counters[2] > 0 else "eager",
             "graph_calls_eager_captured_replayed": list(graph_counters),
             "pool_slots_high_water": max(s["slots_high_water"] for s in st),
         },
