@@ -199,6 +199,38 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     }
 
 
+SWEEP = [
+    # (label, environment of the child).  Any tuning variable routes the launch to the general kernel.
+    ("aligned kernel (default)", {}),
+    ("general kernel, 256 threads x 1 vector", {"IBCOMM_HIP_NO_ALIGNED_KERNEL": "1"}),
+    ("general, 256 x 2", {"IBCOMM_HIP_UNROLL": "2"}),
+    ("general, 256 x 4", {"IBCOMM_HIP_UNROLL": "4"}),
+    ("general, 1024 x 1", {"IBCOMM_HIP_THREADS": "1024"}),
+    ("general, 1024 x 2", {"IBCOMM_HIP_THREADS": "1024", "IBCOMM_HIP_UNROLL": "2"}),
+    ("general, 256 x 1, at most 2048 workgroups (grid-stride)", {"IBCOMM_HIP_MAX_BLOCKS": "2048"}),
+    ("general, 256 x 2, at most 2048 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "2048", "IBCOMM_HIP_UNROLL": "2"}),
+    ("general, 256 x 4, at most 1024 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "1024", "IBCOMM_HIP_UNROLL": "4"}),
+    ("aligned, ordinary loads and stores", {"IBCOMM_HIP_NONTEMPORAL": "0"}),
+    ("aligned, non-temporal loads only", {"IBCOMM_HIP_NONTEMPORAL": "3"}),
+    ("aligned, non-temporal stores only", {"IBCOMM_HIP_NONTEMPORAL": "4"}),
+]
+
+
+def sweep(config):
+    """One child process per variant; nothing here touches the GPU itself."""
+    import subprocess
+    print("%-58s %-28s %10s %10s %8s" % ("variant", "launch shape", "us/launch", "GB/s", "of peak"))
+    for label, env in SWEEP:
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--only-roofline", "--config", str(config)],
+                               env={**os.environ, **env}, capture_output=True, text=True)
+        lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
+        if child.returncode != 0 or not lines:
+            print("%-58s failed (exit %d): %s" % (label, child.returncode, child.stderr.strip().splitlines()[-1:] or ""))
+            continue
+        r = json.loads(lines[-1])["roofline"]
+        print("%-58s %-28s %10.2f %10.1f %8.4f" % (label, r["launch_shape"], r["avg_launch_us"], r["achieved"], r["frac"]), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -212,8 +244,14 @@ def main():
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="run the roofline leg once per kernel variant and launch setting (each in a child process, "
+                         "because the library reads its tuning variables once) and print one line per variant")
     args = ap.parse_args()
 
+    if args.sweep:
+        sweep(args.config)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU only: every emulated rank lives on the same MI355X and nothing in this build "
               "uses a second device; run with --gpus 1", file=sys.stderr)
