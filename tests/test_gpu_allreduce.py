@@ -96,6 +96,7 @@ def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
     # every replay must give what an eager run gives, with other device work in between
     n = 262144 + 3
     with H.World(world_size) as w:
+        w.set_graph_mode(1)  # whatever IBCOMM_HIP_GRAPH says
         w.set_landing(landing)
         w.set_max_fuse(5)
         send = [torch.empty(n, device="cuda") for _ in range(world_size)]
@@ -136,6 +137,7 @@ def test_one_rank_replayed_against_recorded_peers(algo, world_size, chunk, landi
         orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
         assert orc == 0
         with H.World(world_size) as w:
+            w.set_graph_mode(1)  # whatever IBCOMM_HIP_GRAPH says
             w.set_landing(landing)
             send = G.to_device(host)
             recv = [G.poisoned_like(t) for t in send]
