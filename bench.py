@@ -249,6 +249,9 @@ def main():
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
+    ap.add_argument("--whole-buffer", action="store_true",
+                    help="also time the reduction kernel over one whole per-rank buffer in a single segment "
+                         "(roofline.whole_buffer_launch): what it sustains once a launch is large")
     ap.add_argument("--sweep", action="store_true",
                     help="run the roofline leg once per kernel variant and launch setting (each in a child process, "
                          "because the library reads its tuning variables once) and print one line per variant")
@@ -410,10 +413,13 @@ def main():
     }
     if not args.no_roofline:
         line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
-        # the same kernel over one whole per-rank buffer: what it sustains once the launch is large
-        whole = roofline_leg(torch, H, send, recv, n, 1, 40)
-        line["roofline"]["whole_buffer_launch"] = {k: whole[k] for k in (
-            "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
+        if args.whole_buffer:
+            # the same kernel over one whole per-rank buffer: what it sustains once the launch is large.
+            # Not part of the default run, so that a profile of the default run holds the dominant
+            # shape only under this kernel's name.
+            whole = roofline_leg(torch, H, send, recv, n, 1, 40)
+            line["roofline"]["whole_buffer_launch"] = {k: whole[k] for k in (
+                "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
     del recv
     if not args.no_cpu:
         del send
