@@ -2,6 +2,9 @@
 """Benchmark of the MI355X allreduce hot path.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
+    python bench.py --only-roofline [--config N]     the kernel leg alone (what the counter profiles run)
+    python bench.py --whole-buffer                    adds roofline.whole_buffer_launch to the line
+    python bench.py --sweep [--config N]              the kernel leg per kernel variant and launch setting
 
 One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
 collective: every partial sum the rank receives is added to its own contribution (the result going
