@@ -21,7 +21,8 @@
 // is on a 16-byte boundary and every length a whole number of vectors (in practice all of the
 // engine's, since chunk sizes and buffers are aligned): load, add, store, nothing else, because
 // with one vector per lane a workgroup lives for one memory round trip and every instruction ahead
-// of its loads delays them.  SegmentKernel takes everything else (odd offsets, ragged tails, a
+// of its loads delays them; for launches of moderate size it also orders its tiles so that each
+// of the 8 dies works on runs of consecutive tiles.  SegmentKernel takes everything else (odd offsets, ragged tails, a
 // second destination, the tuning experiments).
 //
 // One IEEE-754 add per element, no multiply, so nothing can contract into an
