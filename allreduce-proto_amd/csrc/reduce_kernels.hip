@@ -141,32 +141,42 @@ int EnvInt(const char* name, int fallback) {
   return v ? atoi(v) : fallback;
 }
 
-template <typename T, typename V, int NT, bool XCD>
-hipError_t LaunchAlignedOne(const SegmentBatch& batch, dim3 grid, hipStream_t stream) {
+// The three shapes the aligned kernel is launched in, by vectors in the largest segment.
+enum AlignedShape { kDieLocal256, kPlain256, kPlain128 };
+
+template <typename T, typename V, int NT, int THREADS, bool XCD>
+hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, hipStream_t stream) {
+  const uint64_t blocks = (max_nvec + THREADS - 1) / THREADS;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
   if (batch.seg[0].b != nullptr)
-    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, 256, NT, true, XCD>), grid, dim3(256), 0, stream, batch);
+    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, THREADS, NT, true, XCD>), grid, dim3(THREADS), 0, stream, batch);
   else
-    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, 256, NT, false, XCD>), grid, dim3(256), 0, stream, batch);
+    hipLaunchKernelGGL((AlignedSegmentKernel<T, V, THREADS, NT, false, XCD>), grid, dim3(THREADS), 0, stream, batch);
   return hipGetLastError();
 }
 
-template <typename T, typename V, bool XCD>
-hipError_t LaunchAlignedNT(const SegmentBatch& batch, dim3 grid, int nt, hipStream_t stream) {
-  switch (nt & 7) {
-    case 0: return LaunchAlignedOne<T, V, 0, XCD>(batch, grid, stream);
-    case 1: return LaunchAlignedOne<T, V, 1, XCD>(batch, grid, stream);
-    case 2: return LaunchAlignedOne<T, V, 2, XCD>(batch, grid, stream);
-    case 3: return LaunchAlignedOne<T, V, 3, XCD>(batch, grid, stream);
-    case 4: return LaunchAlignedOne<T, V, 4, XCD>(batch, grid, stream);
-    case 5: return LaunchAlignedOne<T, V, 5, XCD>(batch, grid, stream);
-    case 6: return LaunchAlignedOne<T, V, 6, XCD>(batch, grid, stream);
-    default: return LaunchAlignedOne<T, V, 7, XCD>(batch, grid, stream);
+template <typename T, typename V, int NT>
+hipError_t LaunchAlignedShape(const SegmentBatch& batch, uint64_t max_nvec, AlignedShape shape, hipStream_t stream) {
+  switch (shape) {
+    case kDieLocal256: return LaunchAlignedOne<T, V, NT, 256, true>(batch, max_nvec, stream);
+    case kPlain256: return LaunchAlignedOne<T, V, NT, 256, false>(batch, max_nvec, stream);
+    default: return LaunchAlignedOne<T, V, NT, 128, false>(batch, max_nvec, stream);
   }
 }
 
 template <typename T, typename V>
-hipError_t LaunchAligned(const SegmentBatch& batch, dim3 grid, int nt, bool xcd, hipStream_t stream) {
-  return xcd ? LaunchAlignedNT<T, V, true>(batch, grid, nt, stream) : LaunchAlignedNT<T, V, false>(batch, grid, nt, stream);
+hipError_t LaunchAligned(const SegmentBatch& batch, uint64_t max_nvec, int nt, AlignedShape shape, hipStream_t stream) {
+  switch (nt & 7) {
+    case 0: return LaunchAlignedShape<T, V, 0>(batch, max_nvec, shape, stream);
+    case 1: return LaunchAlignedShape<T, V, 1>(batch, max_nvec, shape, stream);
+    case 2: return LaunchAlignedShape<T, V, 2>(batch, max_nvec, shape, stream);
+    case 3: return LaunchAlignedShape<T, V, 3>(batch, max_nvec, shape, stream);
+    case 4: return LaunchAlignedShape<T, V, 4>(batch, max_nvec, shape, stream);
+    case 5: return LaunchAlignedShape<T, V, 5>(batch, max_nvec, shape, stream);
+    case 6: return LaunchAlignedShape<T, V, 6>(batch, max_nvec, shape, stream);
+    default: return LaunchAlignedShape<T, V, 7>(batch, max_nvec, shape, stream);
+  }
 }
 
 template <typename T, typename V, int THREADS, int UNROLL, int NT>
@@ -247,18 +257,19 @@ hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuni
 
   static const bool fast_path_off = EnvInt("IBCOMM_HIP_NO_ALIGNED_KERNEL", 0) != 0;
   if (misfit == 0 && tuning.threads == 256 && tuning.unroll == 1 && tuning.max_blocks_x == 0 && !fast_path_off) {
-    const uint64_t blocks = (max_n / per_vec + 255) / 256;
-    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
-    // Die-local runs of tiles pay off up to about 8 Mi fp32 per segment (32 MiB per operand) on MI355X:
-    // +3 % at 2 Mi, +1 % at 8 Mi, nothing at 16 Mi, -3 % at 64 Mi.
-    static const uint64_t xcd_max_blocks = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_XCD_RUN_MAX_BLOCKS", 8192));
-    const bool xcd = blocks >= 64 && blocks <= xcd_max_blocks;
+    // Measured on MI355X, per segment of fp32: die-local runs of tiles give +3 % at 2 Mi elements and
+    // +1 % at 8 Mi, nothing at 16 Mi, -3 % at 64 Mi; 128-thread workgroups give nothing up to 16 Mi and
+    // +3 % from 24 Mi on.  The limits are in 256-vector tiles of the largest segment.
+    static const uint64_t xcd_max_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_XCD_RUN_MAX_BLOCKS", 8192));
+    static const uint64_t wg128_min_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_WG128_MIN_BLOCKS", 16385));
+    const uint64_t max_nvec = max_n / per_vec;
+    const uint64_t tiles = (max_nvec + 255) / 256;
+    const AlignedShape shape = (tiles >= 64 && tiles <= xcd_max_tiles) ? kDieLocal256 : (tiles >= wg128_min_tiles ? kPlain128 : kPlain256);
     switch (dtype) {
-      case kF32: return LaunchAligned<float, f32x4>(batch, grid, tuning.nontemporal, xcd, stream);
-      case kI32: return LaunchAligned<uint32_t, u32x4>(batch, grid, tuning.nontemporal, xcd, stream);
-      case kF64: return LaunchAligned<double, f64x2>(batch, grid, tuning.nontemporal, xcd, stream);
-      case kI64: return LaunchAligned<uint64_t, u64x2>(batch, grid, tuning.nontemporal, xcd, stream);
+      case kF32: return LaunchAligned<float, f32x4>(batch, max_nvec, tuning.nontemporal, shape, stream);
+      case kI32: return LaunchAligned<uint32_t, u32x4>(batch, max_nvec, tuning.nontemporal, shape, stream);
+      case kF64: return LaunchAligned<double, f64x2>(batch, max_nvec, tuning.nontemporal, shape, stream);
+      case kI64: return LaunchAligned<uint64_t, u64x2>(batch, max_nvec, tuning.nontemporal, shape, stream);
       default: return hipErrorInvalidValue;
     }
   }

@@ -218,8 +218,9 @@ SWEEP = [
     ("general, 256 x 1, at most 2048 workgroups (grid-stride)", {"IBCOMM_HIP_MAX_BLOCKS": "2048"}),
     ("general, 256 x 2, at most 2048 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "2048", "IBCOMM_HIP_UNROLL": "2"}),
     ("general, 256 x 4, at most 1024 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "1024", "IBCOMM_HIP_UNROLL": "4"}),
-    ("aligned, plain tile order (no die-local runs)", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0"}),
     ("aligned, die-local runs at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000"}),
+    ("aligned, plain order, 256-thread workgroups at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
+    ("aligned, plain order, 128-thread workgroups at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
     ("aligned, ordinary loads and stores", {"IBCOMM_HIP_NONTEMPORAL": "0"}),
     ("aligned, non-temporal loads only", {"IBCOMM_HIP_NONTEMPORAL": "3"}),
     ("aligned, non-temporal stores only", {"IBCOMM_HIP_NONTEMPORAL": "4"}),
