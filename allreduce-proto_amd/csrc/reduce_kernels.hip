@@ -141,8 +141,11 @@ int EnvInt(const char* name, int fallback) {
   return v ? atoi(v) : fallback;
 }
 
-// The three shapes the aligned kernel is launched in, by vectors in the largest segment.
-enum AlignedShape { kDieLocal256, kPlain256, kPlain128 };
+// How the aligned kernel is launched, chosen by the size of the largest segment.
+struct AlignedShape {
+  int threads;     // 256 or 128
+  bool die_local;  // the XCD tile order
+};
 
 template <typename T, typename V, int NT, int THREADS, bool XCD>
 hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, hipStream_t stream) {
@@ -158,11 +161,11 @@ hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, hipStr
 
 template <typename T, typename V, int NT>
 hipError_t LaunchAlignedShape(const SegmentBatch& batch, uint64_t max_nvec, AlignedShape shape, hipStream_t stream) {
-  switch (shape) {
-    case kDieLocal256: return LaunchAlignedOne<T, V, NT, 256, true>(batch, max_nvec, stream);
-    case kPlain256: return LaunchAlignedOne<T, V, NT, 256, false>(batch, max_nvec, stream);
-    default: return LaunchAlignedOne<T, V, NT, 128, false>(batch, max_nvec, stream);
-  }
+  if (shape.threads == 256)
+    return shape.die_local ? LaunchAlignedOne<T, V, NT, 256, true>(batch, max_nvec, stream)
+                           : LaunchAlignedOne<T, V, NT, 256, false>(batch, max_nvec, stream);
+  return shape.die_local ? LaunchAlignedOne<T, V, NT, 128, true>(batch, max_nvec, stream)
+                         : LaunchAlignedOne<T, V, NT, 128, false>(batch, max_nvec, stream);
 }
 
 template <typename T, typename V>
@@ -257,14 +260,17 @@ hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuni
 
   static const bool fast_path_off = EnvInt("IBCOMM_HIP_NO_ALIGNED_KERNEL", 0) != 0;
   if (misfit == 0 && tuning.threads == 256 && tuning.unroll == 1 && tuning.max_blocks_x == 0 && !fast_path_off) {
-    // Measured on MI355X, per segment of fp32: die-local runs of tiles give +3 % at 2 Mi elements and
-    // +1 % at 8 Mi, nothing at 16 Mi, -3 % at 64 Mi; 128-thread workgroups give nothing up to 16 Mi and
-    // +3 % from 24 Mi on.  The limits are in 256-vector tiles of the largest segment.
-    static const uint64_t xcd_max_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_XCD_RUN_MAX_BLOCKS", 8192));
-    static const uint64_t wg128_min_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_WG128_MIN_BLOCKS", 16385));
+    // Measured on MI355X with fp32 (µs per launch of one segment, 256 threads plain / 256 die-local /
+    // 128 die-local / 128 plain): 1 Mi elements 3.40 / 3.42 / 3.68 / 3.74; 2 Mi 5.5 / 5.5 / 5.5 / 6.4;
+    // 4 Mi 9.87 / 9.44 / 9.21 / 10.6; 8 Mi 17.5 / 17.1 / 16.8 / 18.5; 16 Mi 32.7 / 32.3 / 31.7 / 32.4;
+    // 32 Mi 63.3 / 63.3 / 61.0 / 63.1; 64 Mi 125 / 129 / 122.2 / 122.1; 128 Mi 250 / 265 / 248 / 244.
+    // Hence: 256 threads up to 2 Mi elements, 128 beyond; die-local tile order up to 32 Mi elements.
+    // Both limits are in 256-vector tiles (1 Ki fp32) of the largest segment.
+    static const uint64_t wg128_min_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_WG128_MIN_BLOCKS", 2049));
+    static const uint64_t xcd_max_tiles = static_cast<uint64_t>(EnvInt("IBCOMM_HIP_XCD_RUN_MAX_BLOCKS", 32768));
     const uint64_t max_nvec = max_n / per_vec;
     const uint64_t tiles = (max_nvec + 255) / 256;
-    const AlignedShape shape = (tiles >= 64 && tiles <= xcd_max_tiles) ? kDieLocal256 : (tiles >= wg128_min_tiles ? kPlain128 : kPlain256);
+    const AlignedShape shape = {tiles >= wg128_min_tiles ? 128 : 256, tiles >= 64 && tiles <= xcd_max_tiles};
     switch (dtype) {
       case kF32: return LaunchAligned<float, f32x4>(batch, max_nvec, tuning.nontemporal, shape, stream);
       case kI32: return LaunchAligned<uint32_t, u32x4>(batch, max_nvec, tuning.nontemporal, shape, stream);

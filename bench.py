@@ -154,7 +154,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
         "unit": "GB/s",
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get("%d segments x %d fp32" % (k, seg_elems)),
-        "kernel": "ibcomm_hip::AlignedSegmentKernel<float, float4, 256, nontemporal, add>",
+        "kernel": "ibcomm_hip::AlignedSegmentKernel<float, float4, threads and tile order by launch size, nontemporal, add>",
         "launch_shape": "%d segments x %d fp32" % (k, seg_elems),
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
@@ -218,9 +218,10 @@ SWEEP = [
     ("general, 256 x 1, at most 2048 workgroups (grid-stride)", {"IBCOMM_HIP_MAX_BLOCKS": "2048"}),
     ("general, 256 x 2, at most 2048 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "2048", "IBCOMM_HIP_UNROLL": "2"}),
     ("general, 256 x 4, at most 1024 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "1024", "IBCOMM_HIP_UNROLL": "4"}),
-    ("aligned, die-local runs at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000"}),
-    ("aligned, plain order, 256-thread workgroups at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
-    ("aligned, plain order, 128-thread workgroups at any size", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
+    ("aligned, 256 threads, plain tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
+    ("aligned, 256 threads, die-local tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
+    ("aligned, 128 threads, plain tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
+    ("aligned, 128 threads, die-local tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
     ("aligned, ordinary loads and stores", {"IBCOMM_HIP_NONTEMPORAL": "0"}),
     ("aligned, non-temporal loads only", {"IBCOMM_HIP_NONTEMPORAL": "3"}),
     ("aligned, non-temporal stores only", {"IBCOMM_HIP_NONTEMPORAL": "4"}),
