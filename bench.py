@@ -40,7 +40,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # each calibrated against a device copy of known size; the summaries with the commands are under
 # profiles/.  Shapes that have not been measured report null.
 MEASURED_TRAFFIC_BYTES = {
-    "1 segments x 8388608 fp32": 100672646,     # config 2, profiles/segment_kernel_add_ring8_256MiB.md
+    "1 segments x 8388608 fp32": 100681210,     # config 2, profiles/segment_kernel_add_ring8_256MiB.md
     "2 segments x 25165824 fp32": 603978883,    # config 3, profiles/segment_kernel_add_traffic_rabenseifner16_ring8_64KiB_ring32_2GiB.md
     "1 segments x 2097152 fp32": 25180425,      # config 4, same file
     "1 segments x 16777216 fp32": 201346522,    # config 5, same file
