@@ -237,24 +237,27 @@ LaunchTuning DefaultTuning() {
   return t;
 }
 
-hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuning& tuning, hipStream_t stream) {
-  if (batch.count <= 0) return hipSuccess;
-  if (batch.count > kMaxSegments) return hipErrorInvalidValue;
+hipError_t LaunchSegments(const SegmentBatch& given, int dtype, const LaunchTuning& tuning, hipStream_t stream) {
+  if (given.count <= 0) return hipSuccess;
+  if (given.count > kMaxSegments) return hipErrorInvalidValue;
   const size_t es = DTypeSize(dtype);
   if (es == 0) return hipErrorInvalidValue;
 
+  // Empty segments are dropped here (their pointers may be anything); the kernels see the rest.
+  SegmentBatch batch;
+  batch.count = 0;
   uint64_t max_n = 0;
-  const bool add = batch.seg[0].b != nullptr;
   const uint64_t per_vec = 16 / es;
   uintptr_t misfit = 0;  // any low pointer bit, any length remainder, any second destination
-  for (int i = 0; i < batch.count; i++) {
-    const Segment& s = batch.seg[i];
-    if (s.n && (!s.dst || !s.a)) return hipErrorInvalidValue;
-    if ((s.b != nullptr) != add) return hipErrorInvalidValue;  // a launch is all adds or all copies
+  for (int i = 0; i < given.count; i++) {
+    const Segment& s = given.seg[i];
+    if (s.n == 0) continue;
+    if (!s.dst || !s.a) return hipErrorInvalidValue;
+    if (batch.count && (s.b != nullptr) != (batch.seg[0].b != nullptr)) return hipErrorInvalidValue;  // all adds or all copies
     if (s.n > max_n) max_n = s.n;
-    if (s.n)
-      misfit |= ((reinterpret_cast<uintptr_t>(s.dst) | reinterpret_cast<uintptr_t>(s.a) | reinterpret_cast<uintptr_t>(s.b)) & 15) |
-                (s.n % per_vec) | reinterpret_cast<uintptr_t>(s.dst2);
+    misfit |= ((reinterpret_cast<uintptr_t>(s.dst) | reinterpret_cast<uintptr_t>(s.a) | reinterpret_cast<uintptr_t>(s.b)) & 15) |
+              (s.n % per_vec) | reinterpret_cast<uintptr_t>(s.dst2);
+    batch.seg[batch.count++] = s;
   }
   if (max_n == 0) return hipSuccess;
 

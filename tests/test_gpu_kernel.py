@@ -128,6 +128,59 @@ def test_segment_launch_matches_per_segment_results():
     assert H.lib().ibcomm_hip_reduce_segments(H.F32, k + 1, None, None, None, None, None) == H.INVALID_ARGUMENT
 
 
+@pytest.mark.parametrize("n", [1024 * 63 + 4, 1024 * 64, 1024 * 100 + 12, 1024 * 2048, 1024 * 2049 + 8, 1024 * 5000 + 4,
+                               1024 * 8192 + 512, 1024 * 32768, 1024 * 32769 + 16])
+def test_aligned_kernel_geometries(n):
+    # Vector-aligned launches pick their workgroup size and tile order by segment size (256 threads up to
+    # 2048 tiles of 1 Ki fp32, 128 beyond; permuted tile order from 64 up to 32768 tiles).  Every tile must
+    # still be computed exactly once, including those beyond the last whole group of 64 workgroups.
+    g = torch.Generator(device="cuda").manual_seed(n)
+    a = torch.randn(n, device="cuda", generator=g)
+    b = torch.randn(n, device="cuda", generator=g)
+    d = torch.full((n + 256,), float("nan"), device="cuda")
+    torch.cuda.synchronize()
+    assert H.lib().ibcomm_hip_reduce(H.F32, d.data_ptr(), a.data_ptr(), b.data_ptr(), n, None) == 0, H.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(d[:n].view(torch.int32), (a + b).view(torch.int32))
+    assert torch.isnan(d[n:]).all(), "wrote past the end"
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.float64, torch.int64])
+def test_aligned_kernel_geometries_other_types(dtype):
+    code = {torch.int32: H.I32, torch.float64: H.F64, torch.int64: H.I64}[dtype]
+    for n in (512 * 100 + 8, 1024 * 3000 + 4):
+        g = torch.Generator(device="cuda").manual_seed(n)
+        a = torch.randint(-2**31, 2**31 - 1, (n,), device="cuda", generator=g).to(dtype) if dtype != torch.float64 \
+            else torch.randn(n, device="cuda", generator=g, dtype=dtype)
+        b = a.flip(0).clone()
+        d = torch.zeros_like(a)
+        torch.cuda.synchronize()
+        assert H.lib().ibcomm_hip_reduce(code, d.data_ptr(), a.data_ptr(), b.data_ptr(), n, None) == 0, H.last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(d, a + b)
+
+
+def test_aligned_segments_of_different_sizes_share_a_launch():
+    # the grid is sized for the largest segment and the tile order is permuted per group of 64 workgroups:
+    # the smaller segments must come out complete, and nothing may be written beyond any of them
+    sizes = [1024 * 3, 1024 * 200 + 4, 1024 * 70, 0, 1024 * 2100 + 8, 4]
+    k = len(sizes)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    ta = [torch.randn(s, device="cuda", generator=g) for s in sizes]
+    tb = [torch.randn(s, device="cuda", generator=g) for s in sizes]
+    td = [torch.full((s + 64,), float("nan"), device="cuda") for s in sizes]
+    vp = C.c_void_p
+    torch.cuda.synchronize()
+    rc = H.lib().ibcomm_hip_reduce_segments(H.F32, k, (vp * k)(*[t.data_ptr() for t in td]),
+                                            (vp * k)(*[t.data_ptr() for t in ta]), (vp * k)(*[t.data_ptr() for t in tb]),
+                                            (C.c_size_t * k)(*sizes), None)
+    assert rc == 0, H.last_error()
+    torch.cuda.synchronize()
+    for i, s in enumerate(sizes):
+        assert torch.equal(td[i][:s].view(torch.int32), (ta[i] + tb[i]).view(torch.int32)), "segment %d" % i
+        assert torch.isnan(td[i][s:]).all(), "segment %d wrote past its end" % i
+
+
 def test_large_linear_property():
     # 256 MiB operands: compare with torch's own fp32 add on the device (IEEE add, same rounding)
     n = 67108864
