@@ -14,11 +14,13 @@
 // ibcomm/util.h:32-42.  Element types: float, double, 32- and 64-bit integers.
 #pragma once
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 #include <map>
 #include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "ibcomm/util.h"
 #include "ibcomm_hip.h"
@@ -39,6 +41,8 @@ class IBVerbsCommunicator {
   IBVerbsCommunicator& operator=(IBVerbsCommunicator&&) = delete;
 
   ~IBVerbsCommunicator() {
+    for (ibcomm_hip_comm* c : loop_comms_) ibcomm_hip_comm_destroy(c);
+    if (loop_fabric_) ibcomm_hip_fabric_destroy(loop_fabric_);
     if (!comm_) return;
     Registry& reg = registry();
     std::lock_guard<std::mutex> lock(reg.mu);
@@ -62,12 +66,31 @@ class IBVerbsCommunicator {
     Check(ibcomm_hip_comm_create(w.fabric, world_size, &comm_), __LINE__);
     w.users++;
     world_size_ = world_size;
+    static std::atomic<uint16_t> next_id{1};
+    id_ = next_id++;
+    wired_to_.assign(world_size, -1);
   }
 
-  // Queue-pair bring-up (ibverbs_communicator.cpp:286-353) has nothing to exchange in one process.
-  struct ProcessInfo RegisterProcess(int, struct ProcessInfo) { return ProcessInfo{0, 0, 0}; }
-  struct ProcessInfo CreateQueuePair(int) { return ProcessInfo{0, 0, 0}; }
-  void RegisterQueuePair(int, struct ProcessInfo) {}
+  // Queue-pair bring-up (ibverbs_communicator.cpp:286-353).  Between communicators of one process there
+  // is nothing to exchange: ranks find each other through the loopback world.  The information
+  // returned still names the endpoint (this communicator, the peer index the pair stands for), so
+  // that the one wiring the loopback cannot provide by itself keeps working: a communicator
+  // connecting two of its own queue pairs to each other, as the reference's tests/sendrecv_test.cpp
+  // does (pair 1 to pair 0 of the same object: what is sent "to 0" is received "from 1").
+  struct ProcessInfo CreateQueuePair(int dest_rank) {
+    return ProcessInfo{id_, static_cast<uint32_t>(dest_rank), 0};
+  }
+  struct ProcessInfo RegisterProcess(int dest_rank, struct ProcessInfo pinfo) {
+    RegisterQueuePair(dest_rank, pinfo);
+    return CreateQueuePair(dest_rank);
+  }
+  void RegisterQueuePair(int dest_rank, struct ProcessInfo pinfo) {
+    if (pinfo.lid != id_) return;  // a pair of another communicator: the loopback world connects the two
+    if (dest_rank < 0 || dest_rank >= world_size_ || pinfo.qp_n >= static_cast<uint32_t>(world_size_))
+      util::IbcommError(__FILE__, __LINE__, util::IBCOMM_ERROR_CODE::INVALID_ARGUMENT, "queue pair index outside the world");
+    wired_to_[dest_rank] = static_cast<int>(pinfo.qp_n);
+    wired_to_[pinfo.qp_n] = dest_rank;
+  }
   void RegisterMyself(int my_rank) {
     my_rank_ = my_rank;
     Check(ibcomm_hip_comm_register_myself(comm_, my_rank), __LINE__);
@@ -75,23 +98,23 @@ class IBVerbsCommunicator {
 
   // Point-to-point messaging over the loopback (ibverbs_communicator.cpp:371-606); host or device buffers.
   void Send(int dest_rank, const void* buf, size_t len, bool blocking = true) {
-    Check(ibcomm_hip_send(comm_, dest_rank, buf, len, blocking ? 1 : 0), __LINE__);
+    Check(ibcomm_hip_send(Endpoint(dest_rank), dest_rank, buf, len, blocking ? 1 : 0), __LINE__);
   }
   void Recv(int src_rank, void* buf, size_t len, bool blocking = true) {
-    Check(ibcomm_hip_recv(comm_, src_rank, buf, len, blocking ? 1 : 0), __LINE__);
+    Check(ibcomm_hip_recv(Endpoint(src_rank), src_rank, buf, len, blocking ? 1 : 0), __LINE__);
   }
   bool SendPoll(int dest_rank) {
     int done = 0;
-    Check(ibcomm_hip_send_poll(comm_, dest_rank, &done), __LINE__);
+    Check(ibcomm_hip_send_poll(Endpoint(dest_rank), dest_rank, &done), __LINE__);
     return done != 0;
   }
   bool RecvPoll(int src_rank) {
     int done = 0;
-    Check(ibcomm_hip_recv_poll(comm_, src_rank, &done), __LINE__);
+    Check(ibcomm_hip_recv_poll(Endpoint(src_rank), src_rank, &done), __LINE__);
     return done != 0;
   }
-  void SendWait(int dest_rank) { Check(ibcomm_hip_send_wait(comm_, dest_rank), __LINE__); }
-  void RecvWait(int src_rank) { Check(ibcomm_hip_recv_wait(comm_, src_rank), __LINE__); }
+  void SendWait(int dest_rank) { Check(ibcomm_hip_send_wait(Endpoint(dest_rank), dest_rank), __LINE__); }
+  void RecvWait(int src_rank) { Check(ibcomm_hip_recv_wait(Endpoint(src_rank), src_rank), __LINE__); }
   void Bcast(void* buf, size_t len, int root) { Check(ibcomm_hip_bcast(comm_, buf, len, root), __LINE__); }
 
   // Device buffers.  Blocking; every rank of the world must be inside the same call.
@@ -146,6 +169,23 @@ class IBVerbsCommunicator {
                             : IBCOMM_HIP_I64;
   }
 
+  // The communicator a point-to-point call naming `peer` runs on: this one, or, when this object's
+  // queue pair for `peer` is wired to another queue pair of the same object, the private
+  // communicator that plays the rank at the other end of that wire.
+  ibcomm_hip_comm* Endpoint(int peer) {
+    if (my_rank_ >= 0 || peer < 0 || peer >= world_size_ || wired_to_[peer] < 0) return comm_;
+    if (loop_comms_.empty()) {
+      Check(ibcomm_hip_fabric_create(world_size_, &loop_fabric_), __LINE__);
+      for (int r = 0; r < world_size_; r++) {
+        ibcomm_hip_comm* c = nullptr;
+        Check(ibcomm_hip_comm_create(loop_fabric_, world_size_, &c), __LINE__);
+        loop_comms_.push_back(c);
+        Check(ibcomm_hip_comm_register_myself(c, r), __LINE__);
+      }
+    }
+    return loop_comms_[wired_to_[peer]];
+  }
+
   static void Check(int rc, int line) {
     if (rc == 0) return;
     util::IbcommError(__FILE__, line, static_cast<util::IBCOMM_ERROR_CODE>(rc), "%s", ibcomm_hip_last_error());
@@ -154,4 +194,8 @@ class IBVerbsCommunicator {
   ibcomm_hip_comm* comm_ = nullptr;
   int my_rank_ = -1;
   int world_size_ = 0;
+  uint16_t id_ = 0;                          // names this communicator in the ProcessInfo it hands out
+  std::vector<int> wired_to_;                // per queue pair: the queue pair of this object it is connected to, or -1
+  ibcomm_hip_fabric* loop_fabric_ = nullptr; // private world for self-wired queue pairs
+  std::vector<ibcomm_hip_comm*> loop_comms_;
 };
