@@ -50,6 +50,13 @@ def test_rabenseifner_matches_oracle(world_size, fuse, landing):
             G.check_against_oracle(w, H.RABENSEIFNER, rand_bufs(world_size, n, seed=n + 1, scale=1e-2), chunk)
 
 
+@pytest.mark.parametrize("algo,world_size", [(H.RING, 33), (H.RING, 64), (H.RABENSEIFNER, 64), (H.RABENSEIFNER, 128)])
+def test_many_ranks(algo, world_size):
+    with H.World(world_size) as w:
+        G.check_against_oracle(w, algo, rand_bufs(world_size, 300007, seed=world_size, scale=0.1), None)
+        G.check_against_oracle(w, algo, rand_bufs(world_size, 65536 * 4, seed=world_size + 1, scale=0.1), 1024)
+
+
 @pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
 def test_one_thread_per_rank_blocking_calls(algo):
     # the reference's usage: every rank inside its own blocking call at the same time
