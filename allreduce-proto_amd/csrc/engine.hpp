@@ -42,6 +42,7 @@
 #include <chrono>
 #include <deque>
 #include <thread>
+#include <utility>
 #include <vector>
 
 #include "loopback.hpp"
@@ -252,8 +253,8 @@ class Communicator {
     TraceScope scope(&trace_, Trace::kOther);
     int rc = pool_.SynchronizeStreams();
     if (rc == kOk && wait_pulls) {
-      for (Event e : pull_events_) {
-        rc = B::EventSynchronize(e);
+      for (const PullEvent& p : pull_events_) {
+        rc = B::EventSynchronize(p.event);
         if (rc != kOk) break;
       }
     }
@@ -403,6 +404,21 @@ class Communicator {
     size_t len = 0;
     bool active = false;
   };
+  struct PullEvent {
+    Stream stream;
+    Event event;
+  };
+  // A later event on a stream covers the earlier ones, so one event per peer stream is all that
+  // Finish() has to wait for, however many messages the peers pulled.
+  void NotePull(Event e, Stream s) {
+    for (PullEvent& p : pull_events_) {
+      if (p.stream == s) {
+        p.event = e;
+        return;
+      }
+    }
+    pull_events_.push_back(PullEvent{s, e});
+  }
 
   static bool Descending(const Plan& p) { return p.recvs.size() > 1 && p.recvs[1].chunk < p.recvs[0].chunk; }
 
@@ -489,14 +505,22 @@ class Communicator {
     return B::EventRecord(st->event, s);
   }
 
+  // The messages of a batch usually carry one and the same event (their sender produced them with one
+  // launch), and so do the chunks of a group: within one flush a stream waits for an event once.
+  bool WaitedAlready(Stream s, Event e) {
+    for (const auto& w : waited_)
+      if (w.first == s && w.second == e) return true;
+    waited_.emplace_back(s, e);
+    return false;
+  }
   // Orders stream s after `st` unless it already is (same stream) or there is nothing to wait for.
   int WaitOn(Stream s, const OpState& st) {
-    if (!st.has_event || st.stream == s) return kOk;
+    if (!st.has_event || st.stream == s || WaitedAlready(s, st.event)) return kOk;
     stats_.stream_waits++;
     return B::StreamWaitEvent(s, st.event);
   }
   int WaitOnMessage(Stream s, const Message& m) {
-    if (!m.has_ready || m.ready_stream == s) return kOk;
+    if (!m.has_ready || m.ready_stream == s || WaitedAlready(s, m.ready)) return kOk;
     stats_.stream_waits++;
     return B::StreamWaitEvent(s, m.ready);
   }
@@ -512,7 +536,7 @@ class Communicator {
                       (unsigned long long)c.ticket, peer, (unsigned long long)ps.ticket);
         const SendOp& s = plan_.sends[ps.send_index];
         outstanding_sends_--;
-        if (c.has_done) pull_events_.push_back(c.done);
+        if (c.has_done) NotePull(c.done, c.done_stream);
         if (s.dep >= 0 && staged_[s.dep] != nullptr) {
           // the peer has fetched the staged partial sum: the slot is free once its read completes
           if (c.has_done) controller_.returnMemory(staged_[s.dep], c.done, c.done_stream);
@@ -616,6 +640,7 @@ class Communicator {
   // Finished chunks: recvbuf[c] <- message.
   int FlushGathers() {
     if (pending_gather_.empty()) return kOk;
+    waited_.clear();
     TraceScope scope(&trace_, Trace::kIssueCopyKernel);
     if (landing_ != kLandMemcpy) {
       Stream s;
@@ -669,6 +694,7 @@ class Communicator {
   // Partial sums: land every pending message, then one launch adds them all.
   int FlushReduces() {
     if (pending_reduce_.empty()) return kOk;
+    waited_.clear();
     const size_t n = pending_reduce_.size();
     Stream s{};
     std::vector<OpState> landed(n);
@@ -807,7 +833,7 @@ class Communicator {
   }
 
   int WaitOnSlot(Stream s, const Memory<B>* slot) {
-    if (!slot->has_free_event || slot->free_stream == s) return kOk;
+    if (!slot->has_free_event || slot->free_stream == s || WaitedAlready(s, slot->free_event)) return kOk;
     stats_.stream_waits++;
     return B::StreamWaitEvent(s, slot->free_event);
   }
@@ -840,7 +866,8 @@ class Communicator {
   std::vector<std::deque<PostedSend>> posted_;  // per peer: sends awaiting completion, oldest first
   std::vector<PendingRecv> pending_reduce_, pending_gather_;
   int reduce_runs_ = 0, gather_runs_ = 0;  // kernel segments the pending lists will merge into
-  std::vector<Event> pull_events_;
+  std::vector<std::pair<Stream, Event>> waited_;  // (stream, event) pairs already ordered in the current flush
+  std::vector<PullEvent> pull_events_;    // per peer stream: the latest read of this rank's memory enqueued on it
   std::vector<Event> events_[2];
   int arena_ = 0;
   size_t event_cursor_ = 0;
