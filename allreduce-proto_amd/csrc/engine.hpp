@@ -208,6 +208,7 @@ class Communicator {
     chunk_pulled_.assign(chunks, OpState());
     chunk_in_batch_.assign(chunks, 0);
     posted_.assign(world_size_, std::deque<PostedSend>());
+    arrived_.assign(world_size_, std::deque<Message>());
     pending_reduce_.clear();
     pending_gather_.clear();
     // A slot needs spare bytes only if some chunk of recvbuf starts off a 16-byte boundary.  Without
@@ -527,8 +528,13 @@ class Communicator {
 
   int DrainSendCompletions(bool* moved) {
     for (int peer = 0; peer < world_size_; peer++) {
-      typename Fabric<B>::Completion c;
-      while (!posted_[peer].empty() && fabric_->PollSendCompletion(rank_, peer, &c)) {
+      if (posted_[peer].empty()) continue;
+      completions_.clear();
+      fabric_->PollSendCompletions(rank_, peer, &completions_);
+      for (const typename Fabric<B>::Completion& c : completions_) {
+        if (posted_[peer].empty())
+          return Fail(kTransportError, "rank %d: completion for ticket %llu from rank %d with no send outstanding", rank_,
+                      (unsigned long long)c.ticket, peer);
         const PostedSend ps = posted_[peer].front();
         posted_[peer].pop_front();
         if (ps.ticket != c.ticket)
@@ -556,26 +562,38 @@ class Communicator {
     return kOk;
   }
 
+  // Hands the sends collected for one peer to the loopback under one lock.
+  void PostCollected(int peer) {
+    if (out_msgs_.empty()) return;
+    const uint64_t first = fabric_->PostSendBatch(rank_, peer, out_msgs_.data(), out_msgs_.size());
+    for (size_t i = 0; i < out_msgs_.size(); i++) posted_[peer].push_back(PostedSend{first + i, out_index_[i]});
+    out_msgs_.clear();
+    out_index_.clear();
+  }
+
   int PostSends(bool* moved) {
+    int batch_peer = -1;
     while (next_send_ < plan_.sends.size()) {
       const SendOp& s = plan_.sends[next_send_];
-      const void* src;
-      Event ready{};
-      Stream ready_stream{};
-      bool has_ready = false;
+      Message m;
       if (s.dep < 0) {
-        src = SendPtr(s.chunk);
+        m.src = SendPtr(s.chunk);
       } else {
         const OpState& d = recv_done_[s.dep];
         if (!d.issued) break;  // the data has not been enqueued yet
-        src = staged_[s.dep] ? staged_[s.dep]->LandingFor(RecvPtr(s.chunk)) : RecvPtr(s.chunk);
-        ready = d.event;
-        ready_stream = d.stream;
-        has_ready = d.has_event;
+        m.src = staged_[s.dep] ? staged_[s.dep]->LandingFor(RecvPtr(s.chunk)) : RecvPtr(s.chunk);
+        m.ready = d.event;
+        m.ready_stream = d.stream;
+        m.has_ready = d.has_event;
       }
       TraceScope scope(&trace_, Trace::kIssueSend);
-      const uint64_t ticket = fabric_->PostSend(rank_, s.peer, src, ChunkBytes(s.chunk), ready, has_ready, ready_stream);
-      posted_[s.peer].push_back(PostedSend{ticket, static_cast<int>(next_send_)});
+      m.bytes = ChunkBytes(s.chunk);
+      if (s.peer != batch_peer) {
+        PostCollected(batch_peer);
+        batch_peer = s.peer;
+      }
+      out_msgs_.push_back(m);
+      out_index_.push_back(static_cast<int>(next_send_));
       const bool from_staging = s.dep >= 0 && staged_[s.dep] != nullptr;
       if (!from_staging && (s.dep >= 0 || in_place_)) chunk_unconsumed_[s.chunk]++;
       outstanding_sends_++;
@@ -583,7 +601,19 @@ class Communicator {
       next_send_++;
       *moved = true;
     }
+    PostCollected(batch_peer);
     return kOk;
+  }
+
+  // Reports the pulls of a list of messages, all completing with `done`, peer by peer in the order taken.
+  void CompleteAll(const std::vector<PendingRecv>& list, const OpState& done) {
+    size_t i = 0;
+    while (i < list.size()) {
+      const int peer = plan_.recvs[list[i].op].peer;
+      tickets_.clear();
+      while (i < list.size() && plan_.recvs[list[i].op].peer == peer) tickets_.push_back(list[i++].msg.ticket);
+      fabric_->CompleteBatch(rank_, peer, tickets_.data(), tickets_.size(), done.event, true, done.stream);
+    }
   }
 
   int TakeMessages(bool* moved) {
@@ -593,9 +623,13 @@ class Communicator {
       if (r.kind == kGather && chunk_unconsumed_[r.chunk] > 0) break;
       PendingRecv p;
       trace_.Mark(Trace::kReceived);
-      const bool got = fabric_->Take(rank_, r.peer, &p.msg, next_send_);
+      std::deque<Message>& arrived = arrived_[r.peer];  // taken from the loopback, not yet consumed by the plan
+      if (arrived.empty()) fabric_->TakeAll(rank_, r.peer, &arrived, next_send_);
+      const bool got = !arrived.empty();
       if (!got) trace_.Unmark(Trace::kReceived);
       if (!got) break;
+      p.msg = arrived.front();
+      arrived.pop_front();
       trace_.Mark(Trace::kReceived);
       if (p.msg.bytes != ChunkBytes(r.chunk))
         return Fail(kTransportError, "rank %d: message of %zu bytes from rank %d where chunk %d has %zu", rank_, p.msg.bytes,
@@ -660,11 +694,10 @@ class Communicator {
       stats_.gather_copies++;
       OpState done;
       IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+      CompleteAll(pending_gather_, done);
       for (const PendingRecv& p : pending_gather_) {
-        const RecvOp& r = plan_.recvs[p.op];
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
         recv_done_[p.op] = done;
-        chunk_last_[r.chunk] = done;
+        chunk_last_[plan_.recvs[p.op].chunk] = done;
       }
     } else {
       for (const PendingRecv& p : pending_gather_) {
@@ -749,10 +782,7 @@ class Communicator {
         stats_.landing_copies++;
         OpState done;
         IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
-        for (size_t i = 0; i < n; i++) {
-          const PendingRecv& p = pending_reduce_[i];
-          fabric_->Complete(rank_, plan_.recvs[p.op].peer, p.msg.ticket, done.event, true, done.stream);
-        }
+        CompleteAll(pending_reduce_, done);
       }
     }
 
@@ -792,9 +822,9 @@ class Communicator {
       recv_done_[p.op] = done;
       chunk_last_[r.chunk] = done;
       if (p.slot) controller_.returnMemory(p.slot, done.event, s);
-      if (ZeroCopyReceive()) fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
       chunk_in_batch_[r.chunk] = 0;
     }
+    if (ZeroCopyReceive()) CompleteAll(pending_reduce_, done);
     pending_reduce_.clear();
     reduce_runs_ = 0;
     return kOk;
@@ -866,6 +896,11 @@ class Communicator {
   std::vector<std::deque<PostedSend>> posted_;  // per peer: sends awaiting completion, oldest first
   std::vector<PendingRecv> pending_reduce_, pending_gather_;
   int reduce_runs_ = 0, gather_runs_ = 0;  // kernel segments the pending lists will merge into
+  std::vector<std::deque<Message>> arrived_;  // per peer: messages taken from the loopback in one go, oldest first
+  std::vector<typename Fabric<B>::Completion> completions_;  // scratch of DrainSendCompletions
+  std::vector<Message> out_msgs_;         // sends collected for one peer, posted together
+  std::vector<int> out_index_;            // ... and their indices in plan_.sends
+  std::vector<uint64_t> tickets_;         // scratch of CompleteAll
   std::vector<std::pair<Stream, Event>> waited_;  // (stream, event) pairs already ordered in the current flush
   std::vector<PullEvent> pull_events_;    // per peer stream: the latest read of this rank's memory enqueued on it
   std::vector<Event> events_[2];

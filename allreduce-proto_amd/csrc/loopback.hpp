@@ -59,25 +59,39 @@ class Fabric {
 
   uint64_t PostSend(int from, int to, const void* src, size_t bytes, typename B::Event ready, bool has_ready,
                     typename B::Stream ready_stream = typename B::Stream{}) {
-    Channel& c = chan(from, to);
-    std::lock_guard<std::mutex> lock(c.mu);
-    if (from == replay_rank_) {
-      // The peer is a ghost: nobody will read the data, the send is complete at once.
-      Completion k;
-      k.ticket = c.next_ticket++;
-      c.completions.push_back(k);
-      return k.ticket;
-    }
     Message m;
     m.src = src;
     m.bytes = bytes;
     m.ready = ready;
     m.has_ready = has_ready;
     m.ready_stream = ready_stream;
-    m.ticket = c.next_ticket++;
-    c.inbox.push_back(m);
-    c.posted++;
-    return m.ticket;
+    return PostSendBatch(from, to, &m, 1);
+  }
+
+  // Posts n messages (src, bytes and the ready fields filled in) to one peer in one go; their tickets
+  // are consecutive and the first is returned.  One lock per batch instead of one per message matters
+  // when sender and receiver are threads of their own: a receiver that polls takes the same lock.
+  uint64_t PostSendBatch(int from, int to, const Message* msgs, size_t n) {
+    Channel& c = chan(from, to);
+    std::lock_guard<std::mutex> lock(c.mu);
+    const uint64_t first = c.next_ticket;
+    if (from == replay_rank_) {
+      // The peer is a ghost: nobody will read the data, the sends are complete at once.
+      for (size_t i = 0; i < n; i++) {
+        Completion k;
+        k.ticket = c.next_ticket++;
+        c.completions.push_back(k);
+      }
+      return first;
+    }
+    for (size_t i = 0; i < n; i++) {
+      Message m = msgs[i];
+      m.ticket = c.next_ticket++;
+      m.record_to = nullptr;
+      c.inbox.push_back(m);
+    }
+    c.posted += n;
+    return first;
   }
 
   // Receiver: remove and return the oldest message `from` has posted for `to`.  The receiver now
@@ -112,6 +126,28 @@ class Fabric {
     return true;
   }
 
+  // Receiver: all messages `from` has posted for `to` that may be taken now, appended to *out in
+  // order, under one lock (one at a time while recording or replaying, where each message is tied to
+  // the receiver's own progress).  Returns how many were appended.
+  size_t TakeAll(int to, int from, std::deque<Message>* out, size_t sends_posted = 0) {
+    if (to == replay_rank_ || to == record_rank_) {
+      Message m;
+      if (!Take(to, from, &m, sends_posted)) return 0;
+      out->push_back(m);
+      return 1;
+    }
+    Channel& c = chan(from, to);
+    std::lock_guard<std::mutex> lock(c.mu);
+    size_t n = 0;
+    while (!c.inbox.empty() && c.inbox.front().ticket < c.visible_below) {
+      out->push_back(c.inbox.front());
+      c.inbox.pop_front();
+      n++;
+    }
+    c.taken += n;
+    return n;
+  }
+
   // Lockstep emulation for a single-threaded driver.  Real ranks run at the same time, so what a
   // rank can receive at some instant does not depend on the order a driver happens to visit the
   // ranks in.  BeginSweep() freezes, for every channel, the set of receivable messages to those
@@ -133,16 +169,23 @@ class Fabric {
   // Receiver: the pull of message `ticket` has been enqueued; `done` completes when it has read the source.
   void Complete(int to, int from, uint64_t ticket, typename B::Event done, bool has_done,
                 typename B::Stream done_stream = typename B::Stream{}) {
+    CompleteBatch(to, from, &ticket, 1, done, has_done, done_stream);
+  }
+  // The same for n messages of one channel whose pulls share one completion event.
+  void CompleteBatch(int to, int from, const uint64_t* tickets, size_t n, typename B::Event done, bool has_done,
+                     typename B::Stream done_stream = typename B::Stream{}) {
     if (to == replay_rank_) return;  // recorded messages have no sender waiting for them
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
-    Completion k;
-    k.ticket = ticket;
-    k.done = done;
-    k.has_done = has_done;
-    k.done_stream = done_stream;
-    c.completions.push_back(k);
-    c.delivered++;
+    for (size_t i = 0; i < n; i++) {
+      Completion k;
+      k.ticket = tickets[i];
+      k.done = done;
+      k.has_done = has_done;
+      k.done_stream = done_stream;
+      c.completions.push_back(k);
+    }
+    c.delivered += n;
   }
 
   bool PollSendCompletion(int from, int to, Completion* out) {
@@ -152,6 +195,16 @@ class Fabric {
     *out = c.completions.front();
     c.completions.pop_front();
     return true;
+  }
+
+  // Sender: every completion that is there, appended to *out in order, under one lock.
+  size_t PollSendCompletions(int from, int to, std::vector<Completion>* out) {
+    Channel& c = chan(from, to);
+    std::lock_guard<std::mutex> lock(c.mu);
+    const size_t n = c.completions.size();
+    out->insert(out->end(), c.completions.begin(), c.completions.end());
+    c.completions.clear();
+    return n;
   }
 
   // Messages posted but not yet taken, over all channels (0 when idle).
