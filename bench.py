@@ -360,6 +360,19 @@ def main():
                       "parity_bit_exact": copied_ok}
             del out
 
+        # 5. and the most literal form: every message lands in a pool slot through its own hipMemcpyAsync
+        #    (always issued eagerly), unless that is the mode already measured
+        memcpy_landing = None
+        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")) != "memcpy":
+            w.set_landing(H.LAND_MEMCPY)
+            out = torch.empty_like(send[rank])
+            m_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), min(args.steps, 10), 2)
+            m_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
+            parity = parity and m_ok
+            memcpy_landing = {"ms_per_step": round(m_sec * 1e3, 4), "algbw_GBps": round(n * 4 / m_sec * 1e-9, 2),
+                              "parity_bit_exact": m_ok}
+            del out
+
     def device_bytes(s):
         return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
 
@@ -412,6 +425,7 @@ def main():
                 "frac_of_hbm_peak": round(world_bytes / world_sec * 1e-9 / HBM_PEAK_GBPS, 4),
             },
             "rank_with_copy_kernel_landing": copied,
+            "rank_with_hipMemcpyAsync_landing": memcpy_landing,
             "streams_per_rank": st[0]["streams_created"],
             "issue": "hip graph replay" if graph_counters[2] > 0 else "eager",
             "graph_calls_eager_captured_replayed": list(graph_counters),
