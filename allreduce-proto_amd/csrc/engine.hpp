@@ -103,10 +103,10 @@ class Communicator {
   }
 
   // PrepareMemoryPool (ibcomm/ibverbs_communicator_cuda.cpp:26-37) plus this build's knobs.
-  int Init() {
+  int Init(size_t pool_block_bytes = 0) {
     if (world_size_ < 1 || world_size_ != fabric_->world_size())
       return Fail(kInvalidArgument, "world size %d does not match the fabric's %d", world_size_, fabric_->world_size());
-    IBCOMM_RETURN_IF_ERROR(pool_.Init());
+    IBCOMM_RETURN_IF_ERROR(pool_.Init(pool_block_bytes));
     const char* v = getenv("IBCOMM_HIP_MAX_FUSE");
     max_fuse_ = v ? atoi(v) : kMaxSegments;
     if (max_fuse_ < 1 || max_fuse_ > kMaxSegments)

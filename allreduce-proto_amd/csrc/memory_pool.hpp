@@ -105,10 +105,12 @@ class MemoryPool {
   MemoryPool& operator=(const MemoryPool&) = delete;
   ~MemoryPool() { Destroy(); }
 
-  // Reads the knobs and allocates the first block (memory_pool.h:86-100).
-  int Init() {
+  // Reads the knobs and allocates the first block (memory_pool.h:86-100).  A non-zero
+  // `block_bytes` replaces IBCOMM_MEMORY_POOL_PRE_ALLOC (for a backend whose memory is bounded).
+  int Init(size_t block_bytes = 0) {
     IBCOMM_RETURN_IF_ERROR(ReadNumStreams(&max_streams_));
     IBCOMM_RETURN_IF_ERROR(ReadPreAlloc(&block_bytes_));
+    if (block_bytes) block_bytes_ = block_bytes;
     return AllocateBlock(block_bytes_, nullptr);
   }
 

@@ -30,6 +30,7 @@ EXPORTS = [
     "ibcomm_hip_fabric_set_graph_mode", "ibcomm_hip_fabric_graph_counters", "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
     "ibcomm_hip_send", "ibcomm_hip_recv", "ibcomm_hip_send_poll", "ibcomm_hip_recv_poll", "ibcomm_hip_send_wait",
     "ibcomm_hip_recv_wait", "ibcomm_hip_bcast", "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
+    "ibcomm_hip_world_allreduce_noalloc",
 ]
 
 
@@ -67,6 +68,7 @@ def lib():
         for suffix in ("_f32", "_i32"):
             getattr(L, name + suffix).argtypes = [vp, vp, vp, sz]
     L.ibcomm_hip_world_allreduce.argtypes = [C.POINTER(vp), i, i, i, C.POINTER(vp), C.POINTER(vp), sz]
+    L.ibcomm_hip_world_allreduce_noalloc.argtypes = [i, i, i, C.POINTER(vp), C.POINTER(vp), sz, vp]
     L.ibcomm_hip_world_record.argtypes = [C.POINTER(vp), i, i, i, i, C.POINTER(vp), C.POINTER(vp), sz]
     L.ibcomm_hip_replay_allreduce.argtypes = [vp, i, i, vp, vp, sz]
     L.ibcomm_hip_reduce.argtypes = [i, vp, vp, vp, sz, vp]
@@ -124,6 +126,14 @@ def rank_to_chunk(n_ranges, world):
     count = (C.c_int * world)()
     assert lib().ibcomm_hip_rank_to_chunk(n_ranges, world, first, count) == 0
     return [list(range(first[r], first[r] + count[r])) for r in range(world)]
+
+
+def world_allreduce_noalloc(world, algo, dtype, send_ptrs, recv_ptrs, length, stream=None):
+    """The whole-world allreduce that allocates nothing, enqueued on `stream` (a hipStream_t value or
+    None for the default stream); the caller synchronises.  Returns the library's status code."""
+    sp = (C.c_void_p * world)(*send_ptrs)
+    rp = (C.c_void_p * world)(*recv_ptrs)
+    return lib().ibcomm_hip_world_allreduce_noalloc(world, algo, dtype, sp, rp, length, stream)
 
 
 class Plan:

@@ -119,6 +119,20 @@ int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* comm, const int32_t* 
 int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
                                const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
 
+/* ibcomm_hip_world_allreduce for callers that cannot allocate device memory or create streams and
+ * events at the time of the call: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments without the
+ * communicators, same results bit for bit, and `stream` (a hipStream_t, NULL = default stream): all
+ * device work of all world_size ranks is enqueued on that one stream and the call returns without
+ * waiting for it.  Staging slots come out of a 64 MiB array that is part of the library's code
+ * object (one copy per GPU, held until the process ends): a call whose ranks could need more, i.e.
+ * world_size * 2 * (chunks per buffer) * (chunk bytes rounded up to 256) > 64 MiB, returns 1 with a
+ * message and enqueues nothing.  Calls on one GPU share the array: they must not overlap in time
+ * (enqueue them on one stream, or synchronise in between).  The first call on a device looks up the
+ * array's address and should be made outside a capture. */
+int ibcomm_hip_world_allreduce_noalloc(int world_size, int algo, int dtype, const void* const* sendbufs,
+                                       void* const* recvbufs, size_t len_elements, void* stream);
+
 /* One rank's share on its own.  ibcomm_hip_world_record runs the whole world once (like
  * ibcomm_hip_world_allreduce) while keeping, in device memory, every message `rank` receives and the
  * point of its own schedule at which each became available.  ibcomm_hip_replay_allreduce then runs
