@@ -67,6 +67,25 @@ struct HipBackend {
     IBCOMM_HIP_CHECK(hipEventSynchronize(e));
     return kOk;
   }
+  // Timers: events that keep a device timestamp, for the trace's device durations.
+  using Timer = hipEvent_t;
+  static constexpr bool kHasTimers = true;
+  static int TimerCreate(Timer* t) {
+    IBCOMM_HIP_CHECK(hipEventCreate(t));
+    return kOk;
+  }
+  static int TimerDestroy(Timer t) {
+    IBCOMM_HIP_CHECK(hipEventDestroy(t));
+    return kOk;
+  }
+  static int TimerRecord(Timer t, Stream s) {
+    IBCOMM_HIP_CHECK(hipEventRecord(t, s));
+    return kOk;
+  }
+  static int TimerElapsedMs(Timer from, Timer to, float* ms) {
+    IBCOMM_HIP_CHECK(hipEventElapsedTime(ms, from, to));
+    return kOk;
+  }
   // Blocking copy between any two buffers, host or device (point-to-point Send/Recv).
   static int CopySync(void* dst, const void* src, size_t bytes) {
     IBCOMM_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDefault));
@@ -76,20 +95,11 @@ struct HipBackend {
     IBCOMM_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
     return kOk;
   }
-  // `role` says what the launch is for, so that each can carry its own cache hints:
-  // 0 = reduction, 1 = landing copy into a pool slot, 2 = gather into recvbuf.
-  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int role = 0) {
-    LaunchTuning t = DefaultTuning();
-    static const int nt_reduce = EnvMask("IBCOMM_HIP_NT_REDUCE", t.nontemporal);
-    static const int nt_landing = EnvMask("IBCOMM_HIP_NT_LANDING", t.nontemporal);
-    static const int nt_gather = EnvMask("IBCOMM_HIP_NT_GATHER", t.nontemporal);
-    t.nontemporal = role == 0 ? nt_reduce : (role == 1 ? nt_landing : nt_gather);
-    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, t, s));
+  // `role` says what the launch is for (0 = reduction, 1 = landing copy into a pool slot,
+  // 2 = gather into recvbuf); the kernels are the same for all three.
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0) {
+    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, s));
     return kOk;
-  }
-  static int EnvMask(const char* name, int fallback) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : fallback;
   }
 };
 

@@ -2,6 +2,7 @@
 // include/ibcomm_hip.h.
 #include "ibcomm_hip.h"
 
+#include <chrono>
 #include <mutex>
 #include <new>
 #include <string>
@@ -41,6 +42,16 @@ struct CachedGraph {
   hipGraphExec_t exec = nullptr;
 };
 
+// Last node of every recorded graph: counts the replays of a world's graphs in device memory and
+// publishes the count in pinned host memory, where the blocking call that launched the replay is
+// spinning.  Seeing its own count there costs that call a few microseconds less than asking the
+// runtime to synchronise the stream.
+__global__ void PublishReplayCount(uint32_t* count, volatile uint32_t* host_flag) {
+  const uint32_t v = *count + 1;
+  *count = v;
+  *host_flag = v;
+}
+
 struct ibcomm_hip_fabric {
   explicit ibcomm_hip_fabric(int n) : fabric(n) {
     const char* v = getenv("IBCOMM_HIP_GRAPH");
@@ -51,6 +62,10 @@ struct ibcomm_hip_fabric {
   ~ibcomm_hip_fabric() {
     DropGraphs();
     if (origin) (void)hipStreamDestroy(origin);
+    if (replay_count) (void)hipFree(replay_count);
+    if (replay_flag) (void)hipHostFree(replay_flag);
+    if (timer[0]) (void)hipEventDestroy(timer[0]);
+    if (timer[1]) (void)hipEventDestroy(timer[1]);
   }
   void DropGraphs() {
     for (CachedGraph& g : graphs) {
@@ -69,6 +84,11 @@ struct ibcomm_hip_fabric {
   GraphKey last_eager;           // shape of the most recent eagerly issued call
   bool has_last_eager = false;
   uint64_t graph_captures = 0, graph_replays = 0, eager_calls = 0;
+  uint32_t* replay_count = nullptr;  // device: replays of this world's graphs so far (PublishReplayCount)
+  uint32_t* replay_flag = nullptr;   // pinned host memory the last node of a replay writes that count to
+  uint32_t* replay_flag_device = nullptr;
+  uint32_t replays_expected = 0;     // the count the next replay will publish, minus one
+  hipEvent_t timer[2] = {nullptr, nullptr};  // around a replay, when the first communicator traces
 };
 
 struct ibcomm_hip_comm {
@@ -212,9 +232,65 @@ constexpr size_t kMaxCachedGraphs = 16;
 
 uint64_t DeviceOps(const EngineStats& s) { return s.reduce_launches + s.landing_copies + s.gather_copies; }
 
-int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g) {
-  IBCOMM_HIP_CHECK(hipGraphLaunch(g.exec, f->origin));
-  IBCOMM_HIP_CHECK(hipStreamSynchronize(f->origin));
+// Brings the host's idea of the replay count back in line with the device's after a failure.
+void ResyncReplayCount(ibcomm_hip_fabric* f) {
+  (void)hipStreamSynchronize(f->origin);
+  uint32_t v = 0;
+  if (f->replay_count && hipMemcpy(&v, f->replay_count, sizeof v, hipMemcpyDeviceToHost) == hipSuccess) f->replays_expected = v;
+}
+
+// Launches a recorded call and returns when its last node has run.  The wait is a spin on the
+// pinned flag that node writes; if the flag has not come within 20 ms (a long collective, or a
+// device in trouble) the runtime's own wait takes over and reports whatever went wrong.
+int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g, Trace* trace) {
+  const bool traced = trace && trace->enabled();
+  if (traced) {
+    if (!f->timer[0]) IBCOMM_HIP_CHECK(hipEventCreate(&f->timer[0]));
+    if (!f->timer[1]) IBCOMM_HIP_CHECK(hipEventCreate(&f->timer[1]));
+    trace->Mark(Trace::kOther);
+    IBCOMM_HIP_CHECK(hipEventRecord(f->timer[0], f->origin));
+  }
+  const double issued_ms = traced ? trace->NowMs() : 0;
+  const uint32_t expected = f->replays_expected + 1;
+  hipError_t e = hipGraphLaunch(g.exec, f->origin);
+  if (e != hipSuccess) {
+    ResyncReplayCount(f);
+    return Fail(kDeviceError, "hipGraphLaunch failed: %s", hipGetErrorString(e));
+  }
+  f->replays_expected = expected;
+  if (traced) {
+    IBCOMM_HIP_CHECK(hipEventRecord(f->timer[1], f->origin));
+    trace->Mark(Trace::kOther);  // end of the span "graph launched"
+    trace->Mark(Trace::kOther);  // start of the span "waiting for the graph"
+  }
+  const volatile uint32_t* flag = f->replay_flag;
+  const auto t0 = std::chrono::steady_clock::now();
+  bool seen = false;
+  for (uint32_t spins = 1; !seen; spins++) {
+    seen = (*flag == expected);
+    if (!seen && (spins & 0xfff) == 0 &&
+        std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 0.020)
+      break;
+  }
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  // Every so often (and whenever the flag was slow) let the runtime retire what it has queued.
+  if (!seen || (expected & 0x3ff) == 0 || traced) {
+    e = hipStreamSynchronize(f->origin);
+    if (e != hipSuccess) {
+      ResyncReplayCount(f);
+      return Fail(kDeviceError, "hipStreamSynchronize failed after a graph replay: %s", hipGetErrorString(e));
+    }
+    if (*flag != expected) {
+      ResyncReplayCount(f);
+      return Fail(kDeviceError, "a graph replay finished without publishing its completion count (%u, expected %u)", *flag, expected);
+    }
+  }
+  if (traced) {
+    trace->Mark(Trace::kOther);
+    float ms = 0;
+    IBCOMM_HIP_CHECK(hipEventElapsedTime(&ms, f->timer[0], f->timer[1]));
+    trace->AddDevice(Trace::kDeviceGraph, issued_ms, ms);
+  }
   f->graph_replays++;
   return kOk;
 }
@@ -229,6 +305,14 @@ template <class IssueFn>
 int CaptureIssue(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key, IssueFn issue,
                  CachedGraph* out) {
   if (!f->origin) IBCOMM_HIP_CHECK(hipStreamCreateWithFlags(&f->origin, hipStreamNonBlocking));
+  if (!f->replay_count) {
+    IBCOMM_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&f->replay_count), 256));
+    IBCOMM_HIP_CHECK(hipMemset(f->replay_count, 0, 256));
+    IBCOMM_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&f->replay_flag), 64, hipHostMallocMapped));
+    *f->replay_flag = 0;
+    IBCOMM_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&f->replay_flag_device), f->replay_flag, 0));
+    f->replays_expected = 0;
+  }
   for (auto* c : cs) c->pool().OverrideStream(f->origin);
   hipError_t e = hipStreamBeginCapture(f->origin, hipStreamCaptureModeRelaxed);
   int rc = kOk;
@@ -236,6 +320,12 @@ int CaptureIssue(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& c
     rc = Fail(kDeviceError, "hipStreamBeginCapture failed: %s", hipGetErrorString(e));
   } else {
     rc = issue(false);
+    if (rc == kOk) {
+      hipLaunchKernelGGL(PublishReplayCount, dim3(1), dim3(1), 0, f->origin, f->replay_count,
+                         static_cast<volatile uint32_t*>(f->replay_flag_device));
+      const hipError_t le = hipGetLastError();
+      if (le != hipSuccess) rc = Fail(kDeviceError, "recording the completion node failed: %s", hipGetErrorString(le));
+    }
   }
   for (auto* c : cs) c->pool().ClearOverride();
   if (e != hipSuccess) return rc;
@@ -269,7 +359,7 @@ int IssueCached(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs
     return issue(true);
   }
   for (CachedGraph& g : f->graphs)
-    if (g.key == key) return ReplayGraph(f, g);
+    if (g.key == key) return ReplayGraph(f, g, &cs[0]->trace());
 
   if (f->has_last_eager && f->last_eager == key) {
     CachedGraph g;
@@ -287,7 +377,7 @@ int IssueCached(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs
       f->graphs.erase(f->graphs.begin());
     }
     f->graphs.push_back(g);
-    return ReplayGraph(f, f->graphs.back());  // recording executes nothing: run it once
+    return ReplayGraph(f, f->graphs.back(), &cs[0]->trace());  // recording executes nothing: run it once
   }
 
   f->eager_calls++;
@@ -420,9 +510,39 @@ int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, cons
   batch.count = n_segments;
   for (int i = 0; i < n_segments; i++) {
     if (len[i] && (!dst[i] || !a[i] || !b[i])) return Fail(kInvalidArgument, "null operand in segment %d", i);
-    batch.seg[i] = Segment{dst[i], nullptr, a[i], b[i], len[i]};
+    batch.seg[i] = Segment{dst[i], a[i], b[i], len[i]};
   }
-  IBCOMM_HIP_CHECK(LaunchSegments(batch, dtype, DefaultTuning(), static_cast<hipStream_t>(stream)));
+  IBCOMM_HIP_CHECK(LaunchSegments(batch, dtype, static_cast<hipStream_t>(stream)));
+  return kOk;
+}
+
+int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const void* const* src, const size_t* len, void* stream) {
+  if (DTypeSize(dtype) == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+  if (n_segments < 0 || n_segments > kMaxSegments) return Fail(kInvalidArgument, "at most %d segments per launch", kMaxSegments);
+  if (n_segments && (!dst || !src || !len)) return Fail(kInvalidArgument, "null segment table");
+  SegmentBatch batch;
+  batch.count = n_segments;
+  for (int i = 0; i < n_segments; i++) {
+    if (len[i] && (!dst[i] || !src[i])) return Fail(kInvalidArgument, "null operand in segment %d", i);
+    batch.seg[i] = Segment{dst[i], src[i], nullptr, len[i]};
+  }
+  IBCOMM_HIP_CHECK(LaunchSegments(batch, dtype, static_cast<hipStream_t>(stream)));
+  return kOk;
+}
+
+int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, const void* const* a, const void* const* b,
+                               const size_t* len, int* aligned, int* threads, int* die_local) {
+  if (DTypeSize(dtype) == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+  if (n_segments < 0 || n_segments > kMaxSegments) return Fail(kInvalidArgument, "at most %d segments per launch", kMaxSegments);
+  if (n_segments && (!dst || !a || !b || !len)) return Fail(kInvalidArgument, "null segment table");
+  SegmentBatch batch;
+  batch.count = n_segments;
+  for (int i = 0; i < n_segments; i++) batch.seg[i] = Segment{dst[i], a[i], b[i], len[i]};
+  LaunchShape shape;
+  IBCOMM_HIP_CHECK(DescribeLaunch(batch, dtype, &shape));
+  if (aligned) *aligned = shape.aligned ? 1 : 0;
+  if (threads) *threads = shape.threads;
+  if (die_local) *die_local = shape.die_local ? 1 : 0;
   return kOk;
 }
 

@@ -100,6 +100,7 @@ class Communicator {
     controller_.Release();
     for (auto& arena : events_)
       for (auto e : arena) B::EventDestroy(e);
+    for (auto t : timers_) B::TimerDestroy(t);
   }
 
   // PrepareMemoryPool (ibcomm/ibverbs_communicator_cuda.cpp:26-37) plus this build's knobs.
@@ -117,11 +118,18 @@ class Communicator {
     else if (!strcmp(v, "memcpy")) landing_ = kLandMemcpy;
     else if (!strcmp(v, "direct")) landing_ = kLandDirect;
     else return Fail(kInvalidArgument, "IBCOMM_HIP_LANDING must be memcpy, kernel, direct or staged, not '%s'", v);
-    // The working GPU buffer (IBCOMM_WORK_GPU_MEMORY_SIZE, ibverbs_communicator_cuda.cpp:12-33) held
-    // the second operand of the Rabenseifner kernel.  Here that kernel reads the pool slot itself,
-    // so no such buffer is allocated; the variable is still accepted so job scripts keep working.
+    // The working GPU buffer (IBCOMM_WORK_GPU_MEMORY_SIZE, ibverbs_communicator_cuda.cpp:12-37) held
+    // the second operand of the Rabenseifner kernel.  Here that kernel reads the incoming message
+    // where it lies, so no such buffer is allocated.  The variable keeps its meaning as far as a
+    // caller can observe it: read with atoi, unset or -1 is 32 MiB, anything else is taken as given
+    // (text that is no number reads as 0), a size no allocation could satisfy fails as the
+    // reference's cudaMalloc does (CUDA_ERROR), and a size below the chunk size draws the
+    // reference's warning at the first Rabenseifner call (Begin) instead of an error.
     v = getenv("IBCOMM_WORK_GPU_MEMORY_SIZE");
-    work_gpu_memory_size_ = v ? atoll(v) : (32ll << 20);
+    work_gpu_memory_size_ = v ? atoi(v) : -1;
+    if (work_gpu_memory_size_ == -1) work_gpu_memory_size_ = 32ll << 20;
+    if (work_gpu_memory_size_ < 0)
+      return Fail(kDeviceError, "IBCOMM_WORK_GPU_MEMORY_SIZE=%s: no working buffer of that size can be allocated", v);
     v = getenv("IBCOMM_HIP_TRACE");
     trace_.Enable(v && atoi(v) != 0);
     return kOk;
@@ -159,6 +167,8 @@ class Communicator {
   int Begin(int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len_elements) {
     TraceScope scope(&trace_, Trace::kOther);
     if (active_) return Fail(kNotSupported, "an allreduce is already in progress on this communicator");
+    if (fabric_->poisoned())
+      return Fail(kTransportError, "this loopback world was abandoned after an earlier failure (%s); create a new one", fabric_->poison_reason());
     if (rank_ < 0 || rank_ >= world_size_) return Fail(kInvalidArgument, "RegisterMyself has not been called");
     es_ = DTypeSize(dtype);
     if (es_ == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
@@ -215,6 +225,11 @@ class Communicator {
     // them, slots of a chunk size that is a multiple of 256 bytes lie back to back, so chunks that are
     // neighbours in the buffers are neighbours in the pool too and merge into one kernel segment.
     const size_t chunk_bytes = plan_.part.ranges[0].size() * es_;
+    if (algo == kRabenseifner && static_cast<size_t>(work_gpu_memory_size_) < chunk_bytes) {
+      // allreduce_cuda_impl.h:372-385: warn, grow the working buffer to one chunk, carry on
+      Warn("IBCOMM_GPU_WORK_MEMORY_SIZE is smaller than chunk size.\nruntime-reallocation is occured.");
+      work_gpu_memory_size_ = static_cast<long long>(chunk_bytes);
+    }
     const bool phase_margin = (reinterpret_cast<uintptr_t>(recvbuf_) & 15) != 0 || (chunk_bytes & 15) != 0;
     // The ring's queues visit the chunks of a group from the last to the first, the halving windows
     // from the first to the last; the pool hands out its slots in the same direction.
@@ -259,6 +274,7 @@ class Communicator {
         if (rc != kOk) break;
       }
     }
+    if (rc == kOk) rc = ResolveDeviceSpans();
     ReleaseCall();
     return rc;
   }
@@ -281,23 +297,32 @@ class Communicator {
     IBCOMM_RETURN_IF_ERROR(Begin(algo, dtype, sendbuf, recvbuf, len_elements));
     const char* t = getenv("IBCOMM_HIP_TIMEOUT_S");
     const double limit = t ? atof(t) : 120.0;
-    const auto t0 = std::chrono::steady_clock::now();
+    auto last_progress = std::chrono::steady_clock::now();
     bool progressed = false, finished = false;
     for (;;) {
       const int rc = Progress(&progressed, &finished);
       if (rc != kOk) {
+        // What this rank has posted stays in the channels: no later collective may run on them.
+        fabric_->Poison("a rank failed inside an allreduce");
         Abort();
         return rc;
       }
       if (finished) break;
-      if (!progressed) {
-        std::this_thread::yield();
-        const double waited = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-        if (waited > limit) {
-          Abort();
-          return Fail(kTransportError, "rank %d: no peer progress for %.0f s (recv %zu/%zu, send %zu/%zu)", rank_, limit,
-                      next_recv_, plan_.recvs.size(), next_send_, plan_.sends.size());
-        }
+      if (progressed) {
+        last_progress = std::chrono::steady_clock::now();
+        continue;
+      }
+      if (fabric_->poisoned()) {
+        Abort();
+        return Fail(kTransportError, "rank %d: a peer gave up on this allreduce (%s)", rank_, fabric_->poison_reason());
+      }
+      std::this_thread::yield();
+      const double idle = std::chrono::duration<double>(std::chrono::steady_clock::now() - last_progress).count();
+      if (idle > limit) {
+        fabric_->Poison("a rank saw no peer progress within IBCOMM_HIP_TIMEOUT_S");
+        Abort();
+        return Fail(kTransportError, "rank %d: no peer progress for %.0f s (recv %zu/%zu, send %zu/%zu)", rank_, limit,
+                    next_recv_, plan_.recvs.size(), next_send_, plan_.sends.size());
       }
     }
     return Finish(true);
@@ -409,6 +434,10 @@ class Communicator {
     Stream stream;
     Event event;
   };
+  struct DeviceSpan {
+    typename B::Timer start{}, stop{};
+    Trace::DeviceCategory category = Trace::kDeviceReduce;
+  };
   // A later event on a stream covers the earlier ones, so one event per peer stream is all that
   // Finish() has to wait for, however many messages the peers pulled.
   void NotePull(Event e, Stream s) {
@@ -488,6 +517,8 @@ class Communicator {
     if (controller_.active()) stats_.slot_count = controller_.slot_count();
     controller_.Release();
     pull_events_.clear();
+    spans_.clear();
+    timer_cursor_ = 0;
     active_ = false;
   }
 
@@ -524,6 +555,47 @@ class Communicator {
     if (!m.has_ready || m.ready_stream == s || WaitedAlready(s, m.ready)) return kOk;
     stats_.stream_waits++;
     return B::StreamWaitEvent(s, m.ready);
+  }
+
+  // ---- device durations for the trace -------------------------------------------------------------
+  // Only when tracing, only on a backend that keeps time, and never while the launches are being
+  // recorded into a graph (a replay is timed as a whole by its caller).
+  bool DeviceTiming() const { return B::kHasTimers && trace_.enabled() && !pool_.has_override(); }
+  int NextTimer(typename B::Timer* out) {
+    if (timer_cursor_ == timers_.size()) {
+      typename B::Timer t;
+      IBCOMM_RETURN_IF_ERROR(B::TimerCreate(&t));
+      timers_.push_back(t);
+    }
+    *out = timers_[timer_cursor_++];
+    return kOk;
+  }
+  int SpanBegin(Stream s, Trace::DeviceCategory category) {
+    if (!DeviceTiming()) return kOk;
+    DeviceSpan span;
+    span.category = category;
+    IBCOMM_RETURN_IF_ERROR(NextTimer(&span.start));
+    IBCOMM_RETURN_IF_ERROR(NextTimer(&span.stop));
+    if (spans_.empty()) span_origin_ms_ = trace_.NowMs();
+    IBCOMM_RETURN_IF_ERROR(B::TimerRecord(span.start, s));
+    spans_.push_back(span);
+    return kOk;
+  }
+  int SpanEnd(Stream s) {
+    if (!DeviceTiming()) return kOk;
+    return B::TimerRecord(spans_.back().stop, s);
+  }
+  // After the streams have drained: turn the timer pairs of this call into trace entries.
+  int ResolveDeviceSpans() {
+    for (const DeviceSpan& span : spans_) {
+      float since_first = 0, duration = 0;
+      IBCOMM_RETURN_IF_ERROR(B::TimerElapsedMs(spans_.front().start, span.start, &since_first));
+      IBCOMM_RETURN_IF_ERROR(B::TimerElapsedMs(span.start, span.stop, &duration));
+      trace_.AddDevice(span.category, span_origin_ms_ + since_first, duration);
+    }
+    spans_.clear();
+    timer_cursor_ = 0;
+    return kOk;
   }
 
   int DrainSendCompletions(bool* moved) {
@@ -687,10 +759,12 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
         IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
-        AppendSegment(&batch, Segment{RecvPtr(c), nullptr, p.msg.src, nullptr, ChunkElems(c)}, p.joins);
+        AppendSegment(&batch, Segment{RecvPtr(c), p.msg.src, nullptr, ChunkElems(c)}, p.joins);
         stats_.gather_bytes += ChunkBytes(c);
       }
+      IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
       IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 2));
+      IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
       stats_.gather_copies++;
       OpState done;
       IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
@@ -709,7 +783,9 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
         IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
         IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
+        IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
         IBCOMM_RETURN_IF_ERROR(B::CopyAsync(RecvPtr(c), p.msg.src, ChunkBytes(c), s));
+        IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
         stats_.gather_copies++;
         stats_.gather_bytes += ChunkBytes(c);
         OpState done;
@@ -742,7 +818,9 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOnMessage(si, p.msg));
         IBCOMM_RETURN_IF_ERROR(WaitOnSlot(si, p.slot));
         IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, si));
+        IBCOMM_RETURN_IF_ERROR(SpanBegin(si, Trace::kDeviceCopy));
         IBCOMM_RETURN_IF_ERROR(B::CopyAsync(p.slot->LandingFor(RecvPtr(r.chunk)), p.msg.src, ChunkBytes(r.chunk), si));
+        IBCOMM_RETURN_IF_ERROR(SpanEnd(si));
         stats_.landing_copies++;
         stats_.landing_bytes += ChunkBytes(r.chunk);
         IBCOMM_RETURN_IF_ERROR(RecordEvent(si, &landed[i]));
@@ -771,14 +849,18 @@ class Communicator {
             if (Adjacent(q.msg.src, ChunkBytes(qc), p.msg.src, ChunkBytes(c)) == p.joins) joins = p.joins;
           }
           if (joins == 0 && copy.count == kMaxSegments) {
+            IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
             IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
+            IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
             stats_.landing_copies++;
             copy.count = 0;
           }
-          AppendSegment(&copy, Segment{p.slot->LandingFor(RecvPtr(c)), nullptr, p.msg.src, nullptr, ChunkElems(c)}, joins);
+          AppendSegment(&copy, Segment{p.slot->LandingFor(RecvPtr(c)), p.msg.src, nullptr, ChunkElems(c)}, joins);
           stats_.landing_bytes += ChunkBytes(c);
         }
+        IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
         IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
+        IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
         stats_.landing_copies++;
         OpState done;
         IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
@@ -799,10 +881,12 @@ class Communicator {
         IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.stage));
         staged_[p.op] = p.stage;
       }
-      AppendSegment(&batch, Segment{ResultOf(p), nullptr, IncomingOf(p), OwnOf(p), ChunkElems(c)}, p.joins);
+      AppendSegment(&batch, Segment{ResultOf(p), IncomingOf(p), OwnOf(p), ChunkElems(c)}, p.joins);
       stats_.reduce_elements += ChunkElems(c);
     }
+    IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceReduce));
     IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 0));
+    IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
     stats_.reduce_launches++;
     stats_.reduce_segments += n;
     stats_.reduce_kernel_segments += batch.count;
@@ -908,6 +992,10 @@ class Communicator {
   size_t event_cursor_ = 0;
   EngineStats stats_;
   Trace trace_;
+  std::vector<typename B::Timer> timers_;  // created on demand, reused by every traced call
+  size_t timer_cursor_ = 0;
+  std::vector<DeviceSpan> spans_;          // the traced launches of the call in progress
+  double span_origin_ms_ = 0;              // host time at which the first of them was issued
   std::vector<char> p2p_send_pending_;   // per peer: a non-blocking Send awaits its SendPoll/SendWait
   std::vector<PostedRecv> p2p_recv_;     // per peer: the buffer a non-blocking Recv posted
 };

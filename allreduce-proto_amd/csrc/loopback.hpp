@@ -25,9 +25,11 @@
 
 #include <stdint.h>
 
+#include <atomic>
 #include <deque>
 #include <memory>
 #include <mutex>
+#include <string>
 #include <vector>
 
 namespace ibcomm_hip {
@@ -289,6 +291,23 @@ class Fabric {
   }
   ~Fabric() { FreeLog(); }
 
+  // A rank that gives up inside a collective while its peers may still be in it (one thread per
+  // rank) leaves messages and completions behind that no later collective could tell from its own.
+  // It marks the world instead: peers that are waiting stop with a clear error, and every later
+  // collective on this world is refused.
+  void Poison(const char* reason) {
+    std::lock_guard<std::mutex> lock(poison_mu_);
+    if (!poisoned_.load()) {
+      poison_reason_ = reason;
+      poisoned_.store(true);
+    }
+  }
+  bool poisoned() const { return poisoned_.load(); }
+  const char* poison_reason() {
+    std::lock_guard<std::mutex> lock(poison_mu_);
+    return poison_reason_.c_str();
+  }
+
   // Drops everything queued; used when a collective is abandoned after an error.
   void Reset() {
     for (auto& c : channels_) {
@@ -332,6 +351,9 @@ class Fabric {
 
   int n_;
   std::vector<std::unique_ptr<Channel>> channels_;
+  std::atomic<bool> poisoned_{false};
+  std::mutex poison_mu_;
+  std::string poison_reason_;
   int record_rank_ = -1;    // rank whose incoming messages are being logged
   int recorded_rank_ = -1;  // rank the finished log belongs to
   int replay_rank_ = -1;    // rank currently running against the log

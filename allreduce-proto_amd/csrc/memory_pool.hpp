@@ -147,6 +147,7 @@ class MemoryPool {
     has_override_ = true;
   }
   void ClearOverride() { has_override_ = false; }
+  bool has_override() const { return has_override_; }
 
   // Round-robin over at most max_streams() streams, created on first use.
   int NextStream(typename B::Stream* out) {

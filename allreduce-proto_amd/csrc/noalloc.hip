@@ -91,6 +91,15 @@ struct StaticBackend {
   static int EventRecord(Event, Stream) { return kOk; }
   static int StreamWaitEvent(Stream, Event) { return kOk; }
   static int EventSynchronize(Event) { return kOk; }
+  using Timer = int;
+  static constexpr bool kHasTimers = false;
+  static int TimerCreate(Timer*) { return kOk; }
+  static int TimerDestroy(Timer) { return kOk; }
+  static int TimerRecord(Timer, Stream) { return kOk; }
+  static int TimerElapsedMs(Timer, Timer, float* ms) {
+    *ms = 0;
+    return kOk;
+  }
   static int CopySync(void*, const void*, size_t) { return Fail(kNotSupported, "no point-to-point messaging on this backend"); }
   static int CopyAsync(void* dst, const void* src, size_t bytes, Stream s) {
     if (bytes % 4) return Fail(kInvalidArgument, "copy of %zu bytes is not a whole number of elements", bytes);
@@ -98,7 +107,7 @@ struct StaticBackend {
     return kOk;
   }
   static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0) {
-    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, DefaultTuning(), s));
+    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, s));
     return kOk;
   }
 };

@@ -4,26 +4,31 @@
 // (ibcomm/allreduce_cuda_impl.h:24-33: result[i] += value[i], scalar 4-byte
 // accesses, one launch per chunk) with an out-of-place, multi-segment form:
 //
-//     dst[i] = a[i] + b[i]            (and optionally dst2[i] = the same value)
+//     dst[i] = a[i] + b[i]
 //     dst[i] = a[i]                   (b == nullptr: landing / staging copy)
 //
 // One launch takes up to kMaxSegments independent segments, so every chunk
 // that has landed can be reduced by a single launch, and a chunk whose two
 // operands live in different buffers (pool slot + sendbuf) needs no staging
 // copy.  The work is pure HBM streaming: 12 bytes per fp32 element for the
-// two-source add (16 with the second store), 8 for a copy; there is nothing
-// for MFMA or LDS to do.  Each lane moves 16-byte vectors (global_load_dwordx4
-// / global_store_dwordx4), kUnroll of them per operand in flight, and a
-// segment whose three pointers share their 16-byte phase is peeled at head and
-// tail so the body stays vectorised even when a chunk starts at an odd element.
+// two-source add, 8 for a copy; there is nothing for MFMA or LDS to do.  Each
+// lane moves one 16-byte vector per operand (global_load_dwordx4 /
+// global_store_dwordx4), loads with the non-temporal hint, stores written
+// through to the memory-side cache.
 //
 // Two kernels share that contract.  AlignedSegmentKernel takes the launches in which every pointer
 // is on a 16-byte boundary and every length a whole number of vectors (in practice all of the
 // engine's, since chunk sizes and buffers are aligned): load, add, store, nothing else, because
 // with one vector per lane a workgroup lives for one memory round trip and every instruction ahead
 // of its loads delays them; for launches of moderate size it also orders its tiles so that each
-// of the 8 dies works on runs of consecutive tiles.  SegmentKernel takes everything else (odd offsets, ragged tails, a
-// second destination, the tuning experiments).
+// of the 8 dies works on runs of consecutive tiles.  SegmentKernel takes everything else (odd
+// offsets, ragged tails): a segment whose three pointers share their 16-byte phase is peeled at
+// head and tail so the body stays vectorised, any other segment runs element by element.
+//
+// One workgroup per tile and nothing persistent, on purpose: on MI355X the hardware's own
+// in-order workgroup dispatch keeps the addresses in flight in one narrow moving window, and
+// grid-stride, software-pipelined and several-vectors-per-lane forms of the same kernel all
+// measured slower (6 to 10 % at 256 MiB per operand).
 //
 // One IEEE-754 add per element, no multiply, so nothing can contract into an
 // FMA: results are bit-identical to the host's `float` add, provided fp32
@@ -38,19 +43,20 @@
 
 namespace ibcomm_hip {
 
-struct LaunchTuning {
-  int threads;        // workgroup size: 256 or 1024
-  int unroll;         // 16-byte vectors per lane per operand in flight: 1, 2 or 4
-  int max_blocks_x;   // cap on workgroups per segment (grid-stride beyond it); 0 = no cap
-  int nontemporal;    // which accesses stream past the caches: 1 = loads of a, 2 = loads of b, 4 = stores
+// How a launch will be issued, for tests and the benchmark's report.
+struct LaunchShape {
+  bool aligned;    // AlignedSegmentKernel (true) or SegmentKernel (false)
+  int threads;     // workgroup size: 256, or 128 for large aligned segments
+  bool die_local;  // aligned kernel only: tiles ordered so that each die gets runs of 8 consecutive tiles
+  int segments;    // non-empty segments
 };
-
-LaunchTuning DefaultTuning();
 
 // Enqueue one launch covering batch.seg[0..count).  Empty segments are legal; all segments of a
 // launch must be of one kind (every b set: add, every b null: copy).
 // Returns the HIP error of the launch.
-hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, const LaunchTuning& tuning, hipStream_t stream);
+hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, hipStream_t stream);
+// How LaunchSegments would issue this batch, without launching anything.
+hipError_t DescribeLaunch(const SegmentBatch& batch, int dtype, LaunchShape* shape);
 
 // Convenience for a single segment.
 hipError_t LaunchReduce2(void* dst, const void* a, const void* b, size_t n, int dtype, hipStream_t stream);

@@ -6,11 +6,10 @@
 
 namespace ibcomm_hip {
 
-constexpr int kMaxSegments = 64;  // 64 * 40 B of kernel arguments, under the 4 KiB limit
+constexpr int kMaxSegments = 64;  // 64 * 32 B of kernel arguments, under the 4 KiB limit
 
 struct Segment {
   void* dst;        // written
-  void* dst2;       // optional second destination (nullptr = none)
   const void* a;    // first operand (always read)
   const void* b;    // second operand (nullptr = copy)
   uint64_t n;       // elements

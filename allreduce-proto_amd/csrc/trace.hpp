@@ -14,7 +14,16 @@
 //   issue-copy-kernel   a landing copy or a gather was enqueued
 //   issue-redu-kernel   a reduction launch was enqueued
 //   issue-recv          a pool slot was reserved for an incoming message
-//   other               Begin / Finish of a collective
+//   other               Begin / Finish of a collective; in a graph replay, the call that launches
+//                       the graph and the wait for its completion flag
+//
+// Beyond the reference: three more lines in the same format hold DEVICE durations, measured with
+// HIP events on the streams the work ran on:
+//   device-redu-kernel  each reduction launch (eager issue only)
+//   device-copy-kernel  each landing copy and each gather (eager issue only)
+//   device-graph        each replay of a recorded call, first kernel to last
+// Their start times are on the host clock: the moment the first traced launch was issued plus the
+// device time elapsed since that launch began.
 #pragma once
 
 #include <time.h>
@@ -28,6 +37,7 @@ namespace ibcomm_hip {
 class Trace {
  public:
   enum Category { kReceived, kReduced, kIssueSend, kIssueCopyKernel, kIssueReduKernel, kIssueRecv, kOther, kCategories };
+  enum DeviceCategory { kDeviceReduce, kDeviceCopy, kDeviceGraph, kDeviceCategories };
 
   void Enable(bool on) { enabled_ = on; }
   bool enabled() const { return enabled_; }
@@ -48,6 +58,25 @@ class Trace {
 
   size_t pairs(Category c) const { return events_[c].size() / 2; }
 
+  // Milliseconds on the host clock since the timer base (sets the base if there is none yet).
+  double NowMs() {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC_RAW, &ts);
+    if (!has_base_) { base_ = ts; has_base_ = true; }
+    return Millis(base_, ts);
+  }
+  void AddDevice(DeviceCategory c, double start_ms, double duration_ms) {
+    if (!enabled_) return;
+    device_[c].push_back(start_ms);
+    device_[c].push_back(duration_ms);
+  }
+  size_t device_spans(DeviceCategory c) const { return device_[c].size() / 2; }
+  double device_total_ms(DeviceCategory c) const {
+    double t = 0;
+    for (size_t i = 1; i < device_[c].size(); i += 2) t += device_[c][i];
+    return t;
+  }
+
   // DumpTrace, cpp:183-212.
   bool Dump(const std::string& path) const {
     static const char* names[kCategories] = {"received", "reduced", "issue-send", "issue-copy-kernel",
@@ -61,11 +90,18 @@ class Trace {
       for (size_t i = 0; i + 1 < v.size(); i += 2) out << Millis(base_, v[i]) << "," << Millis(v[i], v[i + 1]) << ",";
       out << std::endl;
     }
+    static const char* device_names[kDeviceCategories] = {"device-redu-kernel", "device-copy-kernel", "device-graph"};
+    for (int c = 0; c < kDeviceCategories; c++) {
+      out << device_names[c] << ",";
+      for (double x : device_[c]) out << x << ",";
+      out << std::endl;
+    }
     return true;
   }
 
   void Clear() {
     for (auto& v : events_) v.clear();
+    for (auto& v : device_) v.clear();
   }
 
  private:
@@ -76,6 +112,7 @@ class Trace {
   bool has_base_ = false;
   struct timespec base_ = {};
   std::vector<struct timespec> events_[kCategories];
+  std::vector<double> device_[kDeviceCategories];  // start_ms, duration_ms, start_ms, ...
 };
 
 // Begin/end pair around a scope.

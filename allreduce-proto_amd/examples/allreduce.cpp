@@ -58,6 +58,7 @@ int main(int argc, char* argv[]) {
   std::vector<Rank> ranks(np);
   for (int r = 0; r < np; r++) {
     ranks[r].comm.reset(new IBVerbsCommunicator(np));
+    ranks[r].comm->PrepareMemoryPool();  // public in the reference (ibverbs_communicator.h:116); nothing left to do here
     for (int i = 0; i < np; i++) {  // the bring-up sequence of the reference (:52-77); nothing to exchange here
       if (i == r) ranks[r].comm->RegisterMyself(i);
       else ranks[r].comm->RegisterQueuePair(i, ranks[r].comm->CreateQueuePair(i));

@@ -138,6 +138,11 @@ class IBVerbsCommunicator {
     Check(ibcomm_hip_allreduce_rabenseifner_host(comm_, DType<T>(), sendbuf, recvbuf, len_elements), __LINE__);
   }
 
+  // ibverbs_communicator.h:116-118, ibverbs_communicator_cuda.cpp:26-37.  The reference's Init calls it
+  // to build the staging pool and the working GPU buffer; here the communicator's constructor has
+  // already built the pool (ibcomm_hip_comm_create), so a caller that names it finds nothing left to do.
+  void PrepareMemoryPool() {}
+
   // ibverbs_communicator.cpp:157-216; the trace is recorded when IBCOMM_HIP_TRACE=1.
   void SetTimerBase() { ibcomm_hip_comm_set_timer_base(comm_); }
   void DumpTrace() const { ibcomm_hip_comm_dump_trace(comm_); }

@@ -30,7 +30,7 @@ EXPORTS = [
     "ibcomm_hip_fabric_set_graph_mode", "ibcomm_hip_fabric_graph_counters", "ibcomm_hip_comm_set_max_fuse", "ibcomm_hip_comm_set_landing", "ibcomm_hip_comm_stats", "ibcomm_hip_comm_reset_stats",
     "ibcomm_hip_send", "ibcomm_hip_recv", "ibcomm_hip_send_poll", "ibcomm_hip_recv_poll", "ibcomm_hip_send_wait",
     "ibcomm_hip_recv_wait", "ibcomm_hip_bcast", "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
-    "ibcomm_hip_world_allreduce_noalloc",
+    "ibcomm_hip_world_allreduce_noalloc", "ibcomm_hip_describe_launch", "ibcomm_hip_copy_segments",
 ]
 
 
@@ -73,6 +73,8 @@ def lib():
     L.ibcomm_hip_replay_allreduce.argtypes = [vp, i, i, vp, vp, sz]
     L.ibcomm_hip_reduce.argtypes = [i, vp, vp, vp, sz, vp]
     L.ibcomm_hip_reduce_segments.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), vp]
+    L.ibcomm_hip_copy_segments.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), vp]
+    L.ibcomm_hip_describe_launch.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_split_buffer.argtypes = [sz, sz, i, C.c_char_p, C.POINTER(sz), C.POINTER(sz), i, C.POINTER(i)]
     L.ibcomm_hip_rank_to_chunk.argtypes = [i, i, C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_get_exp_of_two.argtypes = [i]

@@ -4,7 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
     python bench.py --only-roofline [--config N]     the kernel leg alone (what the counter profiles run)
     python bench.py --whole-buffer                    adds roofline.whole_buffer_launch to the line
-    python bench.py --sweep [--config N]              the kernel leg per kernel variant and launch setting
+    python bench.py --sweep [--config N]              every kernel variant of the measurement library at the launch shape
+    python bench.py --ceiling [--config N]            the best variant, the shipped kernel on a large launch, hipMemcpyAsync
+    python bench.py --overlap [--config N]            other ways to issue a schedule of dependent launches, and to wait for it
 
 One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
 collective: every partial sum the rank receives is added to its own contribution (the result going
@@ -23,6 +25,10 @@ Two more legs, both on rank 0 of a one-GPU run:
   cpu_baseline  the CPU oracle's restatement of the reference's AllreduceRing<float> (scalar loop,
                 gcc -O2, one thread per emulated rank) on the same workload, timed on the host.
 The oracle is used only as that baseline and as the checker of the final result.
+
+--sweep, --ceiling and --overlap use libibcomm_hip_bench.so (allreduce-proto_amd/csrc/bench_variants.hip):
+alternative forms of the kernel and probes of other issue schemes, built for measuring only; the default
+run loads it for `roofline.ceiling` (the best of those forms at the launch shape, next to the shipped kernel).
 """
 import argparse
 import ctypes as C
@@ -40,10 +46,11 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # each calibrated against a device copy of known size; the summaries with the commands are under
 # profiles/.  Shapes that have not been measured report null.
 MEASURED_TRAFFIC_BYTES = {
-    "1 segments x 8388608 fp32": 100681210,     # config 2, profiles/segment_kernel_add_ring8_256MiB.md
-    "2 segments x 25165824 fp32": 603978883,    # config 3, profiles/segment_kernel_add_traffic_rabenseifner16_ring8_64KiB_ring32_2GiB.md
-    "1 segments x 2097152 fp32": 25180425,      # config 4, same file
-    "1 segments x 16777216 fp32": 201346522,    # config 5, same file
+    # (launch shape, workgroup size, die-local tile order) of the aligned kernel -> bytes
+    ("1 segments x 8388608 fp32", 128, 1): 100681210,     # config 2, profiles/segment_kernel_add_ring8_256MiB.md
+    ("2 segments x 25165824 fp32", 128, 1): 603978883,    # config 3, profiles/segment_kernel_add_traffic_rabenseifner16_ring8_64KiB_ring32_2GiB.md
+    ("1 segments x 2097152 fp32", 256, 1): 25180425,      # config 4, same file
+    ("1 segments x 16777216 fp32", 128, 1): 201346522,    # config 5, same file
 }
 
 CONFIGS = {
@@ -106,19 +113,20 @@ def check_result(torch, O, H, algo, send, recv, chunk):
     return bool(ok)
 
 
-def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
-    """Average duration of the dominant kernel at its in-schedule launch shape, HIP events on its own stream."""
+def launch_tables(send, recv, seg_elems, k):
+    """Operand tables for launches of k segments x seg_elems: every operand of every segment a distinct
+    range, successive launches walking through all ranks' buffers (several GiB), and no operand that is
+    read was written by an earlier launch, so nothing is served from a cache (a recently written operand
+    would be: stores that carry a coherence scope leave their lines in the 256 MB memory-side cache):
+    a and b come from two ranks' sendbufs at the same offset, dst from a recvbuf."""
     world = len(send)
-    stream = torch.cuda.Stream()
-    k = segs_per_launch
     vp = C.c_void_p
     n = send[0].numel()
     per_buf = max(1, n // seg_elems)
-    # Every operand of every segment is a distinct range, and successive launches walk through
-    # all ranks' buffers (several GiB), so nothing is served from a cache: dst and a come from
-    # rank r's recvbuf / sendbuf, b from another rank's recvbuf at the same offset.
     shapes = []
-    for i in range(world * 2):
+    # enough launches' worth of distinct operands that a pass over the tables reads at least 2 GiB
+    tables = max(world * 2, -(-(2 << 30) // (8 * seg_elems * k)))
+    for i in range(tables):
         dst, a, b = [], [], []
         for j in range(k):
             idx = (i * k + j)
@@ -126,17 +134,15 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
             off = ((idx // world) % per_buf) * seg_elems * 4
             dst.append(recv[r].data_ptr() + off)
             a.append(send[r].data_ptr() + off)
-            b.append(recv[(r + world // 2) % world].data_ptr() + off)
+            b.append(send[(r + world // 2) % world].data_ptr() + off)
         shapes.append(((vp * k)(*dst), (vp * k)(*a), (vp * k)(*b), (C.c_size_t * k)(*([seg_elems] * k))))
-    L = H.lib()
+    return shapes
 
-    def launch(i):
-        d, a, b, ln = shapes[i % len(shapes)]
-        rc = L.ibcomm_hip_reduce_segments(H.F32, k, d, a, b, ln, stream.cuda_stream)
-        assert rc == 0, H.last_error()
 
+def time_launches(torch, stream, launch, launches, warm=5):
+    """Average seconds per launch: HIP events recorded on the stream the launches go to."""
     with torch.cuda.stream(stream):
-        for i in range(5):
+        for i in range(warm):
             launch(i)
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
@@ -145,21 +151,136 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
             launch(i)
         e1.record(stream)
     e1.synchronize()
-    avg_s = e0.elapsed_time(e1) * 1e-3 / launches
+    return e0.elapsed_time(e1) * 1e-3 / launches
+
+
+def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
+    """Average duration of the dominant kernel at its in-schedule launch shape, HIP events on its own stream."""
+    stream = torch.cuda.Stream()
+    k = segs_per_launch
+    shapes = launch_tables(send, recv, seg_elems, k)
+    L = H.lib()
+
+    def launch(i):
+        d, a, b, ln = shapes[i % len(shapes)]
+        rc = L.ibcomm_hip_reduce_segments(H.F32, k, d, a, b, ln, stream.cuda_stream)
+        assert rc == 0, H.last_error()
+
+    avg_s = time_launches(torch, stream, launch, launches)
     algorithmic = 12.0 * seg_elems * k
+    aligned, threads, die_local = C.c_int(), C.c_int(), C.c_int()
+    d, a, b, ln = shapes[0]
+    assert L.ibcomm_hip_describe_launch(H.F32, k, d, a, b, ln, C.byref(aligned), C.byref(threads), C.byref(die_local)) == 0
+    shape = "%d segments x %d fp32" % (k, seg_elems)
     return {
         "bound": "hbm",
         "achieved": round(algorithmic / avg_s * 1e-9, 1),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get("%d segments x %d fp32" % (k, seg_elems)),
-        "kernel": "ibcomm_hip::AlignedSegmentKernel<float, float4, threads and tile order by launch size, nontemporal, add>",
-        "launch_shape": "%d segments x %d fp32" % (k, seg_elems),
+        # counter traffic is known for the kernel geometry it was collected on, and only for that
+        "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value)) if aligned.value else None,
+        "kernel": "ibcomm_hip::%s<float4, %d threads, add, %s tile order>" % (
+            "AlignedSegmentKernel" if aligned.value else "SegmentKernel", threads.value, "die-local" if die_local.value else "plain"),
+        "launch_shape": shape,
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
         "launches_timed": launches,
     }
+
+
+# ---- the measurement library: kernel variants and issue-mode probes --------------------------------
+
+_bench_lib = None
+
+
+def bench_lib():
+    global _bench_lib
+    if _bench_lib is None:
+        path = os.path.join(ROOT, "allreduce-proto_amd", "libibcomm_hip_bench.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s is not built; run __graft_entry__.build()" % path)
+        B = C.CDLL(path)
+        vp, sz, i, dp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)
+        B.ibv_last_error.restype = C.c_char_p
+        B.ibv_variant_name.restype = C.c_char_p
+        B.ibv_variant_name.argtypes = [i]
+        B.ibv_variant_accepts.argtypes = [i, sz]
+        B.ibv_variant_launch.argtypes = [i, vp, vp, vp, sz, vp]
+        B.ibv_probe_chains.argtypes = [i, vp, vp, vp, sz, sz, i, i, i, dp]
+        B.ibv_probe_flags.argtypes = [i, i, vp, vp, vp, sz, sz, i, i, dp, C.POINTER(i)]
+        B.ibv_probe_blocking_call.argtypes = [i, vp, vp, vp, sz, sz, i, i, dp]
+        _bench_lib = B
+    return _bench_lib
+
+
+def variant_times(torch, H, send, recv, total_elems, add, launches=60, passes=3):
+    """Every variant that takes `total_elems` fp32 in one segment, and the shipped kernel on the same
+    operands: -> [(name, seconds per launch)], shipped kernel first.  Each figure is the median of
+    `passes` HIP-event averages over `launches` back-to-back launches; the passes go round all variants,
+    so that a drift of the device over the run touches all of them alike, and a best-of-many is not
+    just the luckiest single measurement."""
+    B = bench_lib()
+    L = H.lib()
+    stream = torch.cuda.Stream()
+    shapes = launch_tables(send, recv, total_elems, 1)
+
+    def shipped(i):
+        d, a, b, ln = shapes[i % len(shapes)]
+        if add:
+            rc = L.ibcomm_hip_reduce_segments(H.F32, 1, d, a, b, ln, stream.cuda_stream)
+        else:
+            rc = L.ibcomm_hip_copy_segments(H.F32, 1, d, a, ln, stream.cuda_stream)
+        assert rc == 0, H.last_error()
+
+    def variant(v):
+        def launch(i):
+            d, a, b, _ = shapes[i % len(shapes)]
+            rc = B.ibv_variant_launch(v, d[0], a[0], b[0] if add else None, total_elems, stream.cuda_stream)
+            assert rc == 0, B.ibv_last_error()
+        return launch
+
+    runners = [("shipped kernel (%s)" % ("ibcomm_hip_reduce_segments" if add else "ibcomm_hip_copy_segments"), shipped)]
+    runners += [(B.ibv_variant_name(v).decode(), variant(v)) for v in range(B.ibv_variant_count()) if B.ibv_variant_accepts(v, total_elems)]
+    samples = [[] for _ in runners]
+    for _ in range(passes):
+        for k, (_, fn) in enumerate(runners):
+            samples[k].append(time_launches(torch, stream, fn, launches))
+    return [(name, sorted(samples[k])[passes // 2]) for k, (name, _) in enumerate(runners)]
+
+
+def ceiling_leg(torch, H, send, recv, seg_elems, segs_per_launch, shipped_us, full=False):
+    """How far the shipped kernel is from the best any measured form of the kernel reaches at this launch
+    size ("the ceiling"), what the shipped kernel sustains once a launch is large, and the runtime's own
+    device-to-device copy as a 1 read : 1 write datum."""
+    total = seg_elems * segs_per_launch
+    times = variant_times(torch, H, send, recv, total, add=True)
+    best = min(times[1:], key=lambda t: t[1])
+    again = times[0][1]
+    out = {
+        "what": "best of %d other forms of dst = a + b (libibcomm_hip_bench.so) on %d fp32 in one segment, same operands, "
+                "median of 3 HIP-event averages over 60 launches each" % (len(times) - 1, total),
+        "best_variant": best[0],
+        "best_variant_us": round(best[1] * 1e6, 2),
+        "shipped_kernel_us_same_pass": round(again * 1e6, 2),
+        "shipped_over_best": round(again / best[1], 4),
+        "best_variant_frac_of_peak": round(12.0 * total / best[1] * 1e-9 / HBM_PEAK_GBPS, 4),
+    }
+    if full:
+        n = send[0].numel()
+        big = roofline_leg(torch, H, send, recv, n, 1, 40)
+        out["shipped_kernel_large_launch"] = {k: big[k] for k in ("launch_shape", "avg_launch_us", "achieved", "frac")}
+        stream = torch.cuda.Stream()
+        world = len(send)
+
+        def memcpy(i):
+            with torch.cuda.stream(stream):
+                recv[i % world].copy_(send[(i + 1) % world], non_blocking=True)
+
+        t = time_launches(torch, stream, memcpy, 40)
+        out["hipMemcpyAsync_device_to_device"] = {"bytes_moved": 8 * n, "us": round(t * 1e6, 2), "GBps_at_8B_per_element": round(8.0 * n / t * 1e-9, 1),
+                                                  "frac_of_peak": round(8.0 * n / t * 1e-9 / HBM_PEAK_GBPS, 4)}
+    return out
 
 
 def cpu_baseline_leg(O, world, n, chunk, algo_name):
@@ -192,11 +313,26 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     cfg1_ok = all(bool(np.array_equal(r.astype(np.int64), exact)) for r in recv1)
     single_n = 64 * 1024 * 1024  # 256 MiB per operand: memory-bound on any host
     single = O.lib().orc_time_reduce_f32(single_n, 3)
+    import subprocess
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), "unknown")
+    except OSError:
+        pass
+    try:
+        gcc = subprocess.run(["gcc", "--version"], capture_output=True, text=True).stdout.splitlines()[0]
+    except (OSError, IndexError):
+        gcc = "unknown"
     return {
         "value": round(n * 4 / t * 1e-9, 3),
         "unit": "GB/s algbw",
         "cores": min(world, os.cpu_count() or 1),
         "kind": "port",
+        "cpu_model": model,
+        "logical_cpus": os.cpu_count() or 1,
+        "pinning": "none (threads placed by the kernel's scheduler)",
+        "compiler": "%s, -O2 (the reference's release flags), scalar loop not vectorised by this gcc" % gcc,
         "sample": "%s, %d ranks x %d fp32, IBCOMM_CHUNKSIZE=%s, whole workload, best of 15 after 1 warm-up, "
                   "one host thread per emulated rank on %d logical CPUs" % (algo_name, world, n, chunk, os.cpu_count() or 1),
         "seconds": round(t, 3),
@@ -207,40 +343,59 @@ def cpu_baseline_leg(O, world, n, chunk, algo_name):
     }
 
 
-SWEEP = [
-    # (label, environment of the child).  Any tuning variable routes the launch to the general kernel.
-    ("aligned kernel (default)", {}),
-    ("general kernel, 256 threads x 1 vector", {"IBCOMM_HIP_NO_ALIGNED_KERNEL": "1"}),
-    ("general, 256 x 2", {"IBCOMM_HIP_UNROLL": "2"}),
-    ("general, 256 x 4", {"IBCOMM_HIP_UNROLL": "4"}),
-    ("general, 1024 x 1", {"IBCOMM_HIP_THREADS": "1024"}),
-    ("general, 1024 x 2", {"IBCOMM_HIP_THREADS": "1024", "IBCOMM_HIP_UNROLL": "2"}),
-    ("general, 256 x 1, at most 2048 workgroups (grid-stride)", {"IBCOMM_HIP_MAX_BLOCKS": "2048"}),
-    ("general, 256 x 2, at most 2048 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "2048", "IBCOMM_HIP_UNROLL": "2"}),
-    ("general, 256 x 4, at most 1024 workgroups", {"IBCOMM_HIP_MAX_BLOCKS": "1024", "IBCOMM_HIP_UNROLL": "4"}),
-    ("aligned, 256 threads, plain tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
-    ("aligned, 256 threads, die-local tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000", "IBCOMM_HIP_WG128_MIN_BLOCKS": "2000000000"}),
-    ("aligned, 128 threads, plain tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "0", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
-    ("aligned, 128 threads, die-local tile order", {"IBCOMM_HIP_XCD_RUN_MAX_BLOCKS": "2000000000", "IBCOMM_HIP_WG128_MIN_BLOCKS": "0"}),
-    ("aligned, ordinary loads and stores", {"IBCOMM_HIP_NONTEMPORAL": "0"}),
-    ("aligned, non-temporal loads only", {"IBCOMM_HIP_NONTEMPORAL": "3"}),
-    ("aligned, non-temporal stores only", {"IBCOMM_HIP_NONTEMPORAL": "4"}),
-]
+def print_variant_table(title, times, bytes_per_launch):
+    print(title)
+    print("%-100s %10s %10s %8s" % ("variant", "us/launch", "GB/s", "of peak"))
+    for name, t in times:
+        print("%-100s %10.2f %10.1f %8.4f" % (name, t * 1e6, bytes_per_launch / t * 1e-9, bytes_per_launch / t * 1e-9 / HBM_PEAK_GBPS), flush=True)
 
 
-def sweep(config):
-    """One child process per variant; nothing here touches the GPU itself."""
-    import subprocess
-    print("%-58s %-28s %10s %10s %8s" % ("variant", "launch shape", "us/launch", "GB/s", "of peak"))
-    for label, env in SWEEP:
-        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--only-roofline", "--config", str(config)],
-                               env={**os.environ, **env}, capture_output=True, text=True)
-        lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
-        if child.returncode != 0 or not lines:
-            print("%-58s failed (exit %d): %s" % (label, child.returncode, child.stderr.strip().splitlines()[-1:] or ""))
-            continue
-        r = json.loads(lines[-1])["roofline"]
-        print("%-58s %-28s %10.2f %10.1f %8.4f" % (label, r["launch_shape"], r["avg_launch_us"], r["achieved"], r["frac"]), flush=True)
+def overlap_leg(torch, send, recv, seg_elems):
+    """Other ways to issue 14 dependent steps of the launch shape (one rank's ring schedule has 14), and to wait for them."""
+    B = bench_lib()
+    n = send[0].numel()
+    region = n * 4
+    ra, rb, rd = send[0].data_ptr(), send[1].data_ptr(), recv[0].data_ptr()
+    steps = 14
+    us = C.c_double()
+    gave_up = C.c_int()
+
+    def chains(mode, k):
+        assert B.ibv_probe_chains(mode, ra, rb, rd, region, seg_elems, steps, k, 20, C.byref(us)) == 0, B.ibv_last_error()
+        return us.value
+
+    def blocking(method, iters=100):
+        assert B.ibv_probe_blocking_call(method, ra, rb, rd, region, seg_elems, steps, iters, C.byref(us)) == 0, B.ibv_last_error()
+        return us.value
+
+    base = chains(0, 1)
+    print("%d dependent steps of dst = a + b on %d fp32 each (%.1f MB of traffic per step), device pace" % (steps, seg_elems, 12e-6 * seg_elems))
+    print("%-96s %10s %10s %8s" % ("how the steps are issued", "us/sched.", "us/step", "of peak"))
+
+    def row(name, t):
+        print("%-96s %10.2f %10.2f %8.4f" % (name, t, t / steps, 12.0 * seg_elems * steps / t * 1e-3 / HBM_PEAK_GBPS), flush=True)
+
+    row("one stream, in-order launches (what the engine issues; a recorded graph is one such chain)", base)
+    row("one stream, launches without the implicit barrier (hipExtAnyOrderLaunch; ignores the dependency)", chains(1, 1))
+    for k in (1, 2, 4, 8):
+        row("HIP graph of kernel nodes, %d parallel chain(s), each 1/%d of every step" % (k, k), chains(2, k))
+    for k in (2, 4):
+        row("%d streams issued eagerly, each 1/%d of every step" % (k, k), chains(3, k))
+    for flags, any_order, name in ((0, 0, "kernel with the counters' operands but neither signal nor wait"),
+                                   (1, 0, "every wave signals its chunk's ready counter (4 chunks per step)"),
+                                   (3, 0, "... and every workgroup waits for the previous step's counter of its chunk"),
+                                   (3, 1, "... the same, launched without the implicit barrier")):
+        assert B.ibv_probe_flags(flags, any_order, ra, rb, rd, region, seg_elems, steps, 10, C.byref(us), C.byref(gave_up)) == 0, B.ibv_last_error()
+        row(name + (" [some waits gave up]" if gave_up.value else ""), us.value)
+    print()
+    null_pace = blocking(6)
+    print("a kernel boundary on one in-order stream: %d empty kernels back to back take %.2f us, %.2f us each" % (steps, null_pace, null_pace / steps))
+    print("one blocking call = issue the %d steps and return when they are done; host wall time per call, minus the device pace above (%.2f us):" % (steps, base))
+    for method, name in ((0, "launches + hipStreamSynchronize"), (1, "launches + spin on hipStreamQuery"),
+                         (2, "launches + a one-thread kernel writing a flag in pinned host memory, host spins on the flag"),
+                         (3, "graph replay + hipStreamSynchronize"), (4, "graph replay + the flag kernel, host spins on the flag")):
+        t = blocking(method)
+        print("    %-100s %8.2f us per call, %6.2f over device pace" % (name, t, t - base), flush=True)
 
 
 def main():
@@ -260,13 +415,14 @@ def main():
                     help="also time the reduction kernel over one whole per-rank buffer in a single segment "
                          "(roofline.whole_buffer_launch): what it sustains once a launch is large")
     ap.add_argument("--sweep", action="store_true",
-                    help="run the roofline leg once per kernel variant and launch setting (each in a child process, "
-                         "because the library reads its tuning variables once) and print one line per variant")
+                    help="time every kernel variant of the measurement library, adds and copies, at the workload's launch shape")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="the best variant at the launch shape, the shipped kernel on a whole-buffer launch, and hipMemcpyAsync")
+    ap.add_argument("--overlap", action="store_true",
+                    help="other ways of issuing the schedule's dependent launches (graph chains, streams, no-barrier launches, "
+                         "ready counters) and of waiting for them")
     args = ap.parse_args()
 
-    if args.sweep:
-        sweep(args.config)
-        return
     if args.gpus != 1:
         print("bench.py measures one GPU only: every emulated rank lives on the same MI355X and nothing in this build "
               "uses a second device; run with --gpus 1", file=sys.stderr)
@@ -330,6 +486,21 @@ def main():
         leg_segments = max(1, st_rank["largest_reduce_kernel_segments"])
         seg_elems = st_rank["largest_reduce_elements"] // leg_segments
 
+        if args.sweep or args.ceiling or args.overlap:
+            total = seg_elems * leg_segments
+            if args.sweep:
+                print_variant_table("dst = a + b, %d fp32 in one segment (12 B per element)" % total,
+                                    variant_times(torch, H, send, recv, total, True), 12.0 * total)
+                print()
+                print_variant_table("dst = a (the gather and landing copies), %d fp32 in one segment (8 B per element)" % total,
+                                    variant_times(torch, H, send, recv, total, False), 8.0 * total)
+            if args.ceiling:
+                leg = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+                print(json.dumps({"config": args.config, "roofline": leg,
+                                  "ceiling": ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], full=True)}))
+            if args.overlap:
+                overlap_leg(torch, send, recv, total)
+            return
         if args.only_roofline:
             # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
             # counters collected over this command can be calibrated against a known traffic
@@ -339,7 +510,10 @@ def main():
             print(json.dumps({"only_roofline": True, "config": args.config,
                               "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)}))
             return
-        sec_per_step = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
+        # the C entry point with its arguments converted once, as any caller in a loop would hold them
+        replay_fn = H.lib().ibcomm_hip_replay_allreduce
+        replay_args = (w.comms[rank], C.c_int(algo), C.c_int(H.F32), C.c_void_p(sp[rank]), C.c_void_p(out.data_ptr()), C.c_size_t(n))
+        sec_per_step = timed(lambda: replay_fn(*replay_args), args.steps, warm)
         parity = parity and bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
         del out
 
@@ -426,6 +600,8 @@ def main():
             },
             "rank_with_copy_kernel_landing": copied,
             "rank_with_hipMemcpyAsync_landing": memcpy_landing,
+            "north_star_landing_mode": "memcpy (rank_with_hipMemcpyAsync_landing is that mode's figure; `value` is the '%s' mode)" % (
+                args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")),
             "streams_per_rank": st[0]["streams_created"],
             "issue": "hip graph replay" if graph_counters[2] > 0 else "eager",
             "graph_calls_eager_captured_replayed": list(graph_counters),
@@ -434,6 +610,7 @@ def main():
     }
     if not args.no_roofline:
         line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+        line["roofline"]["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, line["roofline"]["avg_launch_us"])
         if args.whole_buffer:
             # the same kernel over one whole per-rank buffer: what it sustains once the launch is large.
             # Not part of the default run, so that a profile of the default run holds the dominant
@@ -446,6 +623,8 @@ def main():
         del send
         torch.cuda.empty_cache()
         line["cpu_baseline"] = cpu_baseline_leg(O, world, n, chunk, algo_name)
+        # the like-for-like GPU figure for that baseline: all N ranks' schedules on the one GPU per step
+        line["cpu_baseline"]["gpu_all_ranks_on_one_gpu_algbw_GBps"] = round(world_algbw, 2)
     print(json.dumps(line))
     if not parity:
         sys.exit(1)

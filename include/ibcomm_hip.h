@@ -163,6 +163,17 @@ int ibcomm_hip_reduce(int dtype, void* dst, const void* a, const void* b, size_t
 int ibcomm_hip_reduce_segments(int dtype, int n_segments, void* const* dst, const void* const* a,
                                const void* const* b, const size_t* len_elements, void* stream);
 int ibcomm_hip_max_segments(void);
+/* The copy launch of the engine on its own: dst[i] = src[i] over several segments, asynchronous on
+ * `stream`.  Stands for the per-chunk cudaMemcpyAsync calls around the reference's kernel
+ * (ibcomm/allreduce_cuda_impl.h:129-130 and :528-529 into recvbuf, :503-504 into the working buffer). */
+int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const void* const* src,
+                             const size_t* len_elements, void* stream);
+/* How ibcomm_hip_reduce_segments would issue these segments, without launching: *aligned = 1 for the
+ * kernel that takes 16-byte aligned pointers and whole vectors (0: the general kernel), *threads the
+ * workgroup size, *die_local = 1 if tiles are ordered in runs per accelerator die.  Stands for the
+ * launch geometry the reference fixes at ibcomm/allreduce_cuda_impl.h:24, 116-117. */
+int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, const void* const* a, const void* const* b,
+                               const size_t* len_elements, int* aligned, int* threads, int* die_local);
 
 /* ---- point-to-point messaging over the loopback ------------------------------------------------ */
 

@@ -194,7 +194,6 @@ class Sim {
         out->push_back(Access{reinterpret_cast<uintptr_t>(s.a), reinterpret_cast<uintptr_t>(s.a) + b, false, i});
         if (s.b) out->push_back(Access{reinterpret_cast<uintptr_t>(s.b), reinterpret_cast<uintptr_t>(s.b) + b, false, i});
         out->push_back(Access{reinterpret_cast<uintptr_t>(s.dst), reinterpret_cast<uintptr_t>(s.dst) + b, true, i});
-        if (s.dst2) out->push_back(Access{reinterpret_cast<uintptr_t>(s.dst2), reinterpret_cast<uintptr_t>(s.dst2) + b, true, i});
       }
     }
   }
@@ -202,14 +201,12 @@ class Sim {
   template <typename T>
   static void RunSegment(const Segment& s) {
     T* d = static_cast<T*>(s.dst);
-    T* d2 = static_cast<T*>(s.dst2);
     const T* a = static_cast<const T*>(s.a);
     const T* b = static_cast<const T*>(s.b);
     for (uint64_t i = 0; i < s.n; i++) {
       T v = a[i];
       if (b) v = v + b[i];
       d[i] = v;
-      if (d2) d2[i] = v;
     }
   }
 
@@ -284,6 +281,15 @@ struct SimBackend {
   }
   static int EventSynchronize(Event) {
     Sim::Get().RunAll();
+    return 0;
+  }
+  using Timer = int;  // the simulated device keeps no time
+  static constexpr bool kHasTimers = false;
+  static int TimerCreate(Timer*) { return 0; }
+  static int TimerDestroy(Timer) { return 0; }
+  static int TimerRecord(Timer, Stream) { return 0; }
+  static int TimerElapsedMs(Timer, Timer, float* ms) {
+    *ms = 0;
     return 0;
   }
   static int CopySync(void* dst, const void* src, size_t bytes) {

@@ -48,3 +48,12 @@ def test_library_errors_end_the_process_with_the_reference_codes():
     assert rc == 1
     rc, _, _ = run(4, "bogus", 4096)
     assert rc == 1
+
+
+def test_the_example_names_every_public_call_of_the_bring_up():
+    # PrepareMemoryPool() is public in the reference's class under USE_CUDA (ibverbs_communicator.h:116):
+    # the example calls it, so the binary that the tests above ran was compiled against a header that has it
+    src = open(os.path.join(ROOT, "allreduce-proto_amd", "examples", "allreduce.cpp")).read()
+    assert "->PrepareMemoryPool()" in src
+    hdr = open(os.path.join(ROOT, "allreduce-proto_amd", "ibcomm", "ibverbs_communicator.h")).read()
+    assert "void PrepareMemoryPool()" in hdr

@@ -62,6 +62,16 @@ def test_bcast_one_thread_per_rank():
             assert torch.equal(bufs[r], torch.full((4096,), 2.0, device="cuda"))
 
 
+TRACE_NAMES = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
+DEVICE_NAMES = ["device-redu-kernel", "device-copy-kernel", "device-graph"]
+
+
+def read_trace(path):
+    lines = open(path).read().splitlines()
+    assert [ln.split(",")[0] for ln in lines] == TRACE_NAMES + DEVICE_NAMES  # the reference's seven lines first
+    return {ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in lines}
+
+
 def test_trace_files(tmp_path):
     base = str(tmp_path / "trace")
     with G.env(IBCOMM_TRACE_FILE=base, IBCOMM_CHUNKSIZE=None):
@@ -72,13 +82,47 @@ def test_trace_files(tmp_path):
             recv = [torch.empty_like(t) for t in send]
             assert G.run_world(w, H.RING, send, recv) == 0
             w.dump_trace()
-    names = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
     for r in range(4):
-        lines = open("%s_%d.dat" % (base, r)).read().splitlines()
-        assert [ln.split(",")[0] for ln in lines] == names
-        received = [float(x) for x in lines[0].split(",")[1:-1]]
+        t = read_trace("%s_%d.dat" % (base, r))
+        received = t["received"]
         assert len(received) == 2 * 2 * 3 * 4  # (start, duration) x 2(N-1) groups x 4 chunks
         assert all(d >= 0 for d in received[1::2])
+        # device durations, one HIP-event pair per launch: N-1 reductions and N-1 gathers per rank, eagerly issued
+        assert len(t["device-redu-kernel"]) == 2 * 3 and len(t["device-copy-kernel"]) == 2 * 3 and t["device-graph"] == []
+        for name in ("device-redu-kernel", "device-copy-kernel"):
+            assert all(0 < d < 50 for d in t[name][1::2]), t[name]        # milliseconds, positive, sane
+            assert t[name][0::2] == sorted(t[name][0::2])                   # launches of one rank follow one another
+        assert len(t["issue-redu-kernel"]) == len(t["device-redu-kernel"])  # one host issue span per device span
+
+
+def test_trace_of_graph_replays(tmp_path):
+    # Every call leaves records: the first is issued eagerly, the second records the graph and replays
+    # it, the others replay.  A replay does no host-side pipeline work; what it leaves is two "other"
+    # spans (the launch call, the wait for the completion flag) and one device-graph duration.
+    base = str(tmp_path / "replay")
+    calls = 6
+    with G.env(IBCOMM_TRACE_FILE=base, IBCOMM_CHUNKSIZE=None):
+        with H.World(4) as w:
+            w.set_graph_mode(1)
+            w.set_trace(True)
+            send = [torch.randn(1 << 18, device="cuda") for _ in range(4)]
+            recv = [torch.empty_like(t) for t in send]
+            want = None
+            for _ in range(calls):
+                assert G.run_world(w, H.RING, send, recv) == 0
+                if want is None:
+                    want = [t.clone() for t in recv]
+                assert all(G.bits_equal(a, b) for a, b in zip(recv, want))
+            assert w.graph_counters() == (1, 1, calls - 1)
+            w.dump_trace()
+    t0 = read_trace(base + "_0.dat")
+    assert len(t0["device-graph"]) == 2 * (calls - 1)
+    assert all(0 < d < 50 for d in t0["device-graph"][1::2])
+    assert len(t0["device-redu-kernel"]) == 2 * 3  # the eager first call only; recording a graph times nothing
+    # Begin and Finish of the eager call and of the recorded one, then two spans per replay
+    assert len(t0["other"]) == 2 * (2 + 1 + 2 * (calls - 1)), len(t0["other"])
+    t1 = read_trace(base + "_1.dat")
+    assert t1["device-graph"] == []  # the replay belongs to the world; it is booked on rank 0's trace
 
 
 @pytest.mark.parametrize("algo,oracle_algo,world_size", [(H.RING, 0, 4), (H.RING, 0, 3), (H.RABENSEIFNER, 1, 4), (H.RABENSEIFNER, 1, 8)])
