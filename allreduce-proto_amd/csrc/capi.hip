@@ -42,14 +42,13 @@ struct CachedGraph {
   hipGraphExec_t exec = nullptr;
 };
 
-// Last node of every recorded graph: counts the replays of a world's graphs in device memory and
-// publishes the count in pinned host memory, where the blocking call that launched the replay is
-// spinning.  Seeing its own count there costs that call a few microseconds less than asking the
-// runtime to synchronise the stream.
-__global__ void PublishReplayCount(uint32_t* count, volatile uint32_t* host_flag) {
-  const uint32_t v = *count + 1;
-  *count = v;
-  *host_flag = v;
+// Last node of every recorded graph: stores the device's wall clock into pinned host memory, where
+// the blocking call that launched the replay is spinning until the word changes.  Seeing the new
+// value costs that call a few microseconds less than asking the runtime to synchronise the stream,
+// and a clock reading needs no state on the device: replays of one world never overlap (each call
+// waits for its own), and two readings that far apart always differ.
+__global__ void PublishCompletion(uint64_t* host_flag) {
+  __hip_atomic_store(host_flag, static_cast<uint64_t>(wall_clock64()), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 struct ibcomm_hip_fabric {
@@ -62,7 +61,6 @@ struct ibcomm_hip_fabric {
   ~ibcomm_hip_fabric() {
     DropGraphs();
     if (origin) (void)hipStreamDestroy(origin);
-    if (replay_count) (void)hipFree(replay_count);
     if (replay_flag) (void)hipHostFree(replay_flag);
     if (timer[0]) (void)hipEventDestroy(timer[0]);
     if (timer[1]) (void)hipEventDestroy(timer[1]);
@@ -84,10 +82,9 @@ struct ibcomm_hip_fabric {
   GraphKey last_eager;           // shape of the most recent eagerly issued call
   bool has_last_eager = false;
   uint64_t graph_captures = 0, graph_replays = 0, eager_calls = 0;
-  uint32_t* replay_count = nullptr;  // device: replays of this world's graphs so far (PublishReplayCount)
-  uint32_t* replay_flag = nullptr;   // pinned host memory the last node of a replay writes that count to
-  uint32_t* replay_flag_device = nullptr;
-  uint32_t replays_expected = 0;     // the count the next replay will publish, minus one
+  uint64_t* replay_flag = nullptr;   // pinned host memory the last node of a replay writes the device clock to
+  uint64_t* replay_flag_device = nullptr;
+  uint64_t replays_issued = 0;
   hipEvent_t timer[2] = {nullptr, nullptr};  // around a replay, when the first communicator traces
 };
 
@@ -232,16 +229,9 @@ constexpr size_t kMaxCachedGraphs = 16;
 
 uint64_t DeviceOps(const EngineStats& s) { return s.reduce_launches + s.landing_copies + s.gather_copies; }
 
-// Brings the host's idea of the replay count back in line with the device's after a failure.
-void ResyncReplayCount(ibcomm_hip_fabric* f) {
-  (void)hipStreamSynchronize(f->origin);
-  uint32_t v = 0;
-  if (f->replay_count && hipMemcpy(&v, f->replay_count, sizeof v, hipMemcpyDeviceToHost) == hipSuccess) f->replays_expected = v;
-}
-
 // Launches a recorded call and returns when its last node has run.  The wait is a spin on the
-// pinned flag that node writes; if the flag has not come within 20 ms (a long collective, or a
-// device in trouble) the runtime's own wait takes over and reports whatever went wrong.
+// pinned word that node writes; if it has not changed within 20 ms (a long collective, or a device
+// in trouble) the runtime's own wait takes over and reports whatever went wrong.
 int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g, Trace* trace) {
   const bool traced = trace && trace->enabled();
   if (traced) {
@@ -251,39 +241,33 @@ int ReplayGraph(ibcomm_hip_fabric* f, CachedGraph& g, Trace* trace) {
     IBCOMM_HIP_CHECK(hipEventRecord(f->timer[0], f->origin));
   }
   const double issued_ms = traced ? trace->NowMs() : 0;
-  const uint32_t expected = f->replays_expected + 1;
+  const volatile uint64_t* flag = f->replay_flag;
+  const uint64_t before = *flag;  // no replay of this world is in flight: nothing writes the word until this one ends
+  f->replays_issued++;
   hipError_t e = hipGraphLaunch(g.exec, f->origin);
   if (e != hipSuccess) {
-    ResyncReplayCount(f);
+    (void)hipStreamSynchronize(f->origin);
     return Fail(kDeviceError, "hipGraphLaunch failed: %s", hipGetErrorString(e));
   }
-  f->replays_expected = expected;
   if (traced) {
     IBCOMM_HIP_CHECK(hipEventRecord(f->timer[1], f->origin));
     trace->Mark(Trace::kOther);  // end of the span "graph launched"
     trace->Mark(Trace::kOther);  // start of the span "waiting for the graph"
   }
-  const volatile uint32_t* flag = f->replay_flag;
   const auto t0 = std::chrono::steady_clock::now();
   bool seen = false;
   for (uint32_t spins = 1; !seen; spins++) {
-    seen = (*flag == expected);
+    seen = (*flag != before);
     if (!seen && (spins & 0xfff) == 0 &&
         std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 0.020)
       break;
   }
   __atomic_thread_fence(__ATOMIC_ACQUIRE);
   // Every so often (and whenever the flag was slow) let the runtime retire what it has queued.
-  if (!seen || (expected & 0x3ff) == 0 || traced) {
+  if (!seen || (f->replays_issued & 0x3ff) == 0 || traced) {
     e = hipStreamSynchronize(f->origin);
-    if (e != hipSuccess) {
-      ResyncReplayCount(f);
-      return Fail(kDeviceError, "hipStreamSynchronize failed after a graph replay: %s", hipGetErrorString(e));
-    }
-    if (*flag != expected) {
-      ResyncReplayCount(f);
-      return Fail(kDeviceError, "a graph replay finished without publishing its completion count (%u, expected %u)", *flag, expected);
-    }
+    if (e != hipSuccess) return Fail(kDeviceError, "hipStreamSynchronize failed after a graph replay: %s", hipGetErrorString(e));
+    if (*flag == before) return Fail(kDeviceError, "a graph replay finished without publishing its completion");
   }
   if (traced) {
     trace->Mark(Trace::kOther);
@@ -305,13 +289,10 @@ template <class IssueFn>
 int CaptureIssue(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, const GraphKey& key, IssueFn issue,
                  CachedGraph* out) {
   if (!f->origin) IBCOMM_HIP_CHECK(hipStreamCreateWithFlags(&f->origin, hipStreamNonBlocking));
-  if (!f->replay_count) {
-    IBCOMM_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&f->replay_count), 256));
-    IBCOMM_HIP_CHECK(hipMemset(f->replay_count, 0, 256));
+  if (!f->replay_flag) {
     IBCOMM_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&f->replay_flag), 64, hipHostMallocMapped));
     *f->replay_flag = 0;
     IBCOMM_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&f->replay_flag_device), f->replay_flag, 0));
-    f->replays_expected = 0;
   }
   for (auto* c : cs) c->pool().OverrideStream(f->origin);
   hipError_t e = hipStreamBeginCapture(f->origin, hipStreamCaptureModeRelaxed);
@@ -321,8 +302,7 @@ int CaptureIssue(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& c
   } else {
     rc = issue(false);
     if (rc == kOk) {
-      hipLaunchKernelGGL(PublishReplayCount, dim3(1), dim3(1), 0, f->origin, f->replay_count,
-                         static_cast<volatile uint32_t*>(f->replay_flag_device));
+      hipLaunchKernelGGL(PublishCompletion, dim3(1), dim3(1), 0, f->origin, f->replay_flag_device);
       const hipError_t le = hipGetLastError();
       if (le != hipSuccess) rc = Fail(kDeviceError, "recording the completion node failed: %s", hipGetErrorString(le));
     }

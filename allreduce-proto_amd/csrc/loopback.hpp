@@ -308,13 +308,17 @@ class Fabric {
     return poison_reason_.c_str();
   }
 
-  // Drops everything queued; used when a collective is abandoned after an error.
+  // Drops everything queued and lifts the mark above; for the owner of the world, once every rank
+  // has left the collective that was abandoned.
   void Reset() {
     for (auto& c : channels_) {
       std::lock_guard<std::mutex> lock(c->mu);
       c->inbox.clear();
       c->completions.clear();
     }
+    std::lock_guard<std::mutex> lock(poison_mu_);
+    poisoned_.store(false);
+    poison_reason_.clear();
   }
 
  private:

@@ -69,10 +69,10 @@ int main(int argc, char** argv) {
   }
   unsetenv("IBCOMM_CHUNKSIZE");
   unsetenv("IBCOMM_MEMORY_POOL_PRE_ALLOC");
-  const int failures_held = extras ? sim_failures() : 1023, p2p_held = extras ? sim_p2p() : 2047;
-  if (failures_held != 1023 || p2p_held != 2047) {
+  const int failures_held = extras ? sim_failures() : 4095, p2p_held = extras ? sim_p2p() : 2047;
+  if (failures_held != 4095 || p2p_held != 2047) {
     bad++;
-    printf("failure-handling checks %d of 1023, point-to-point checks %d of 2047\n", failures_held, p2p_held);
+    printf("failure-handling checks %d of 4095, point-to-point checks %d of 2047\n", failures_held, p2p_held);
   }
   printf("runs %d bad %d\n", runs, bad);
   return bad != 0;

@@ -1,5 +1,8 @@
 // C entry points that run the allreduce engine on the simulated device (see sim_backend.hpp).
 // TEST INFRASTRUCTURE ONLY.
+#include <string.h>
+
+#include <chrono>
 #include <memory>
 #include <string>
 #include <thread>
@@ -92,12 +95,38 @@ int sim_failures(void) {
     const int rc = c0.AllreduceBlocking(kRing, kF32, a.data(), ra.data(), a.size());
     unsetenv("IBCOMM_HIP_TIMEOUT_S");
     if (rc == kTransportError && !c0.active()) held |= 1;
+    // what that rank had posted is still in the channels: the world refuses further collectives ...
+    if (fabric.poisoned() && c1.Begin(kRing, kF32, b.data(), rb.data(), a.size()) == kTransportError &&
+        strstr(LastErrorBuffer(), "abandoned") != nullptr)
+      held |= 1024;
     fabric.Reset();
-    // ... and the communicator is usable afterwards
+    // ... until its owner resets it; then the communicators are usable again
     const void* sends[2] = {a.data(), b.data()};
     void* recvs[2] = {ra.data(), rb.data()};
     Communicator<SimBackend>* cs[2] = {&c0, &c1};
     if (RunWorld<SimBackend>(cs, 2, kRing, kF32, sends, recvs, a.size(), true) == kOk && ra[7] == 3.0f && rb[4095] == 3.0f) held |= 2;
+  }
+  {
+    // three ranks, one never joins: the first to lose patience (0.3 s) marks the world, and the other
+    // stops waiting at once instead of sitting out its own, much longer, time limit (30 s)
+    Fabric<SimBackend> fabric(3);
+    Communicator<SimBackend> c0(&fabric, 3), c1(&fabric, 3);
+    c0.Init(); c1.Init();
+    c0.RegisterMyself(0); c1.RegisterMyself(1);
+    std::vector<float> rc_buf(4096);
+    int r0 = 0, r1 = 0;
+    std::string m1;
+    const auto t0 = std::chrono::steady_clock::now();
+    setenv("IBCOMM_HIP_TIMEOUT_S", "0.3", 1);
+    std::thread t([&]() { r0 = c0.AllreduceBlocking(kRing, kF32, a.data(), ra.data(), a.size()); });
+    std::this_thread::sleep_for(std::chrono::milliseconds(100));  // rank 0 has read its limit by now
+    setenv("IBCOMM_HIP_TIMEOUT_S", "30", 1);
+    r1 = c1.AllreduceBlocking(kRing, kF32, b.data(), rb.data(), b.size());
+    m1 = LastErrorBuffer();
+    t.join();
+    unsetenv("IBCOMM_HIP_TIMEOUT_S");
+    const double took = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (r0 == kTransportError && r1 == kTransportError && took < 5.0 && m1.find("gave up") != std::string::npos) held |= 2048;
   }
   {
     // ranks that disagree about the buffer length: the first mismatching message is a transport error

@@ -321,6 +321,38 @@ def test_pool_knobs_and_single_controller_rule():
     assert pool_rules(IBCOMM_HIP_LANDING="direct")[0] == 0
 
 
+def test_working_gpu_memory_knob(capfd):
+    # IBCOMM_WORK_GPU_MEMORY_SIZE (ibverbs_communicator_cuda.cpp:12-37): atoi, -1 / unset = 32 MiB, anything
+    # else as given; smaller than a chunk -> the reference's warning at a Rabenseifner call and the call
+    # goes on (allreduce_cuda_impl.h:372-385); a size nothing could allocate -> CUDA_ERROR (3).
+    import os
+    world, n = 4, 4096
+    bufs = rand_bufs(world, n, seed=11)
+    rc, base, _ = S.allreduce(RABEN, bufs, 1024)
+    assert rc == 0
+    capfd.readouterr()
+    warning = "IBCOMM_GPU_WORK_MEMORY_SIZE is smaller than chunk size."
+    cases = [("1", True), ("1023", True), ("1024", False), ("garbage", True), ("0", True), ("-1", False), ("33554432", False)]
+    try:
+        for value, warns in cases:
+            os.environ["IBCOMM_WORK_GPU_MEMORY_SIZE"] = value
+            for algo in (RABEN, RING):
+                want = base if algo == RABEN else S.allreduce(RING, bufs, 1024, max_fuse=1)[1]
+                capfd.readouterr()
+                rc, got, rep = S.allreduce(algo, bufs, 1024)
+                err = capfd.readouterr().err
+                assert rc == 0 and rep.races == 0, (value, rep.error)
+                assert all(np.array_equal(O.bits(g), O.bits(w)) for g, w in zip(got, want)), value
+                assert (warning in err) == (warns and algo == RABEN), (value, algo, err)
+                if warning in err:
+                    assert err.count(warning) == world and "runtime-reallocation is occured." in err  # once per rank
+        os.environ["IBCOMM_WORK_GPU_MEMORY_SIZE"] = "-5"
+        rc, _, rep = S.allreduce(RABEN, bufs, 1024)
+        assert rc == 3 and b"IBCOMM_WORK_GPU_MEMORY_SIZE" in rep.error
+    finally:
+        os.environ.pop("IBCOMM_WORK_GPU_MEMORY_SIZE", None)
+
+
 def test_trace_file_has_the_reference_format(tmp_path):
     # ibcomm/ibverbs_communicator.cpp:157-212: seven lines "name,start_ms,dur_ms,...", scientific notation
     import ctypes as C
@@ -344,7 +376,10 @@ def test_trace_file_has_the_reference_format(tmp_path):
     assert rc == 0
     lines = open(path).read().splitlines()
     names = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
-    assert [ln.split(",")[0] for ln in lines] == names
+    # the reference's seven lines, then this build's device-duration lines (empty: the simulated device keeps no time)
+    assert [ln.split(",")[0] for ln in lines] == names + ["device-redu-kernel", "device-copy-kernel", "device-graph"]
+    assert lines[7:] == ["device-redu-kernel,", "device-copy-kernel,", "device-graph,"]
+    lines = lines[:7]
     q = n * 4 // 1024 // world  # chunks per group
     want_pairs = {"received": 2 * (world - 1) * q, "reduced": (world - 1) * q, "issue-send": 2 * (world - 1) * q,
                   "issue-redu-kernel": (world - 1) * q, "issue-recv": (world - 1) * q, "other": 2}
@@ -376,7 +411,8 @@ def test_failure_handling_is_reported_not_hung():
     held = S.lib().sim_failures()
     names = ["missing peer times out", "usable after a timeout", "length mismatch", "second collective refused",
              "p2p refused during a collective", "bad arguments", "replay without recording", "replay of another rank",
-             "replay of another call", "replay still works"]
+             "replay of another call", "replay still works", "an abandoned world refuses collectives until reset",
+             "a waiting peer stops when another rank gives up"]
     missing = [n for k, n in enumerate(names) if not held >> k & 1]
     assert not missing, missing
 

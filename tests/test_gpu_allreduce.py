@@ -367,6 +367,40 @@ def test_config_5_ring_32_ranks_2gib_ragged_tail():
     torch.cuda.empty_cache()
 
 
+def test_config_5_pool_on_the_receive_path_with_4_gib_blocks():
+    # The staging pool at the size 288 GB of HBM allows: one 4 GiB block per rank (four times the ceiling
+    # the reference puts on IBCOMM_MEMORY_POOL_PRE_ALLOC, memory_pool.h:163), and every partial sum a rank
+    # receives landing in a slot of its pool through the copy kernel before it is reduced ("kernel"
+    # landing), at the full size of config 5.  In place, so that 64 GiB of buffers and 128 GiB of pools
+    # fit side by side; the inputs are generated again afterwards to check the result against.
+    world_size, n, chunk = 32, 536870911, 16777216
+    free, _ = torch.cuda.mem_get_info()
+    if free < 215 * 2**30:
+        pytest.skip("needs ~200 GiB of free HBM")
+    with G.env(IBCOMM_MEMORY_POOL_PRE_ALLOC=4 << 30):
+        with H.World(world_size) as w:
+            w.set_landing(H.LAND_KERNEL)
+            bufs = device_inputs(world_size, n, 500, "normal")
+            assert G.run_world(w, H.RING, bufs, bufs, chunk) == 0, H.last_error()
+            stats = [w.stats(r) for r in range(world_size)]
+    torch.cuda.empty_cache()
+    reduced_chunks = (world_size - 1) * 4  # 31 ring steps of one group of 4 chunks
+    for r, s in enumerate(stats):
+        assert s["pool_blocks"] == 1 and s["pool_bytes"] == 4 << 30, r
+        assert s["slot_count"] == 256  # 4 GiB carved into 16 MiB slots, none wasted (the reference's strict '<' would leave 255)
+        assert 4 <= s["slots_high_water"] <= 8, s["slots_high_water"]  # one ring step's chunks, reused first-in first-out
+        assert s["reduce_segments"] == reduced_chunks
+        # every received partial sum went through the pool; the group that holds the ragged tail is the last one
+        assert s["landing_bytes"] in (reduced_chunks * chunk, reduced_chunks * chunk - 4), r
+        assert s["landing_copies"] == world_size - 1
+    send = device_inputs(world_size, n, 500, "normal")
+    check_ring_on_device(send, bufs, chunk)
+    check_stripes_against_oracle(send, bufs[0], H.RING, chunk, [0, 63, 127])
+    check_stripes_against_oracle(send, bufs[31], H.RING, chunk, [127])
+    del send, bufs
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("algo,world_size", [(H.RING, 3), (H.RABENSEIFNER, 2)])
 def test_more_than_2_to_the_31_elements(algo, world_size):
     # The reference indexes chunk ranges with int (ibverbs_communicator.cpp:676-677) and stops short of
@@ -408,3 +442,27 @@ def test_config_1_values_cpu_shape_on_gpu():
         exact = sum(t.double() for t in send).float()
         for r in range(world_size):
             assert torch.equal(recv[r], exact)
+
+
+def test_working_gpu_memory_knob_on_the_device(capfd):
+    # IBCOMM_WORK_GPU_MEMORY_SIZE (ibverbs_communicator_cuda.cpp:12-37, allreduce_cuda_impl.h:372-385): read when
+    # a communicator is created; whatever it says the results are the oracle's, a value below the chunk size
+    # draws the reference's warning at a Rabenseifner call and nothing else, a size no allocation could
+    # satisfy ends the communicator's creation with CUDA_ERROR (3) as the reference's cudaMalloc would.
+    world, n, chunk = 4, 65536, 4096
+    bufs = rand_bufs(world, n, seed=77, scale=1e-2)
+    warning = "IBCOMM_GPU_WORK_MEMORY_SIZE is smaller than chunk size."
+    for value, warns in [("1", True), ("4095", True), ("4096", False), ("not a number", True), (None, False)]:
+        with G.env(IBCOMM_WORK_GPU_MEMORY_SIZE=value):
+            with H.World(world) as w:
+                for algo in (H.RABENSEIFNER, H.RING):
+                    capfd.readouterr()
+                    G.check_against_oracle(w, algo, bufs, chunk)
+                    err = capfd.readouterr().err
+                    assert (warning in err) == (warns and algo == H.RABENSEIFNER), (value, algo, err)
+                capfd.readouterr()
+                G.check_against_oracle(w, H.RABENSEIFNER, bufs, chunk)  # the buffer has "grown": no second warning
+                assert warning not in capfd.readouterr().err
+    with G.env(IBCOMM_WORK_GPU_MEMORY_SIZE="-4096"):
+        with pytest.raises(RuntimeError, match="comm_create: 3 .*IBCOMM_WORK_GPU_MEMORY_SIZE"):
+            H.World(world)

@@ -195,3 +195,52 @@ def test_large_linear_property():
     # and a sampled stripe against the oracle on the host
     s = slice(n - 100003, n)
     assert np.array_equal(O.bits(d[s].cpu().numpy()), O.bits(oracle_add(a[s].cpu().numpy(), b[s].cpu().numpy())))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.float64, np.int64])
+def test_copy_segments_all_widths_and_phases(dtype):
+    # the engine's copy launch on its own (ibcomm_hip_copy_segments): aligned one-segment kernel, aligned
+    # table kernel (several segments) and the general kernel (odd offsets, ragged lengths), for 4- and 8-byte elements
+    rng = np.random.default_rng(3)
+    es = np.dtype(dtype).itemsize
+    dt = O.DTYPE_OF[np.dtype(dtype)]
+    for lens, offs in [([262144], [0]), ([4096, 65536, 16], [0, 0, 0]), ([1000, 3, 70001], [1, 0, 3]), ([0, 5, 0], [0, 1, 0])]:
+        k = len(lens)
+        src = [torch.from_numpy((rng.standard_normal(n + 8) * 100).astype(dtype)).cuda() for n in lens]
+        dst = [torch.zeros(n + 8, dtype=src[0].dtype, device="cuda") for n in lens]
+        for t in dst:
+            t.view(torch.uint8).fill_(0xAB)
+        vp = C.c_void_p
+        d = (vp * k)(*[t.data_ptr() + o * es for t, o in zip(dst, offs)])
+        a = (vp * k)(*[t.data_ptr() + o * es for t, o in zip(src, offs)])
+        ln = (C.c_size_t * k)(*lens)
+        torch.cuda.synchronize()
+        assert H.lib().ibcomm_hip_copy_segments(dt, k, d, a, ln, None) == 0, H.last_error()
+        torch.cuda.synchronize()
+        for t_src, t_dst, n, o in zip(src, dst, lens, offs):
+            got, want = t_dst.cpu().numpy(), t_src.cpu().numpy()
+            assert np.array_equal(O.bits(got[o:o + n]), O.bits(want[o:o + n]))
+            raw = got.view(np.uint8)
+            assert (raw[:o * es] == 0xAB).all() and (raw[(o + n) * es:] == 0xAB).all(), "wrote outside the segment"
+
+
+def test_one_segment_launch_and_table_launch_give_the_same_bits():
+    # a launch of one segment takes its operands as plain kernel arguments, several segments go through the
+    # table: the same data through both, and through the reference's association (one add per element)
+    n = 1 << 20
+    rng = np.random.default_rng(8)
+    a = rng.standard_normal(n).astype(np.float32)
+    b = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    want = oracle_add(a, b)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    one = torch.zeros(n, device="cuda")
+    two = torch.zeros(n, device="cuda")
+    vp = C.c_void_p
+    L = H.lib()
+    assert L.ibcomm_hip_reduce_segments(H.F32, 1, (vp * 1)(one.data_ptr()), (vp * 1)(ta.data_ptr()), (vp * 1)(tb.data_ptr()),
+                                        (C.c_size_t * 1)(n), None) == 0
+    h = n // 2
+    assert L.ibcomm_hip_reduce_segments(H.F32, 2, (vp * 2)(two.data_ptr(), two.data_ptr() + 4 * h), (vp * 2)(ta.data_ptr(), ta.data_ptr() + 4 * h),
+                                        (vp * 2)(tb.data_ptr(), tb.data_ptr() + 4 * h), (C.c_size_t * 2)(h, h), None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(O.bits(one.cpu().numpy()), O.bits(want)) and np.array_equal(O.bits(two.cpu().numpy()), O.bits(want))

@@ -123,3 +123,40 @@ def test_baseline_config_plan_shapes():
     p = H.Plan(H.RING, 32, 31, 536870911, 4, 16777216)
     assert len(p.ranges) == 128 and p.ranges[-1] == (127 * 4194304, 536870911)
     assert len(p.recvs) == 2 * 31 * 4
+
+
+def test_launch_geometry_follows_the_segment_size():
+    # ibcomm_hip_describe_launch touches no device: how a launch would be issued is decided on the host.
+    # The reference fixes 512 threads and min(ceil(n / 512), 65535) blocks for every size
+    # (allreduce_cuda_impl.h:24, 116-117); here the aligned kernel runs one 16-byte vector per lane,
+    # 256-thread workgroups up to 2 Mi fp32 per segment and 128 beyond, die-local tile order from 64 tiles
+    # up to 32 Mi fp32, and anything off the 16-byte grid goes to the general kernel.
+    import ctypes as C
+    L = H.lib()
+
+    def describe(lens, dtype=H.F32, base=(0x10000000, 0x20000000, 0x30000000)):
+        k = len(lens)
+        vp = C.c_void_p
+        d = (vp * k)(*[base[0] + i * 0x1000000 for i in range(k)])
+        a = (vp * k)(*[base[1] + i * 0x1000000 for i in range(k)])
+        b = (vp * k)(*[base[2] + i * 0x1000000 for i in range(k)])
+        ln = (C.c_size_t * k)(*lens)
+        al, th, dl = C.c_int(-1), C.c_int(-1), C.c_int(-1)
+        assert L.ibcomm_hip_describe_launch(dtype, k, d, a, b, ln, C.byref(al), C.byref(th), C.byref(dl)) == 0, H.last_error()
+        return al.value, th.value, dl.value
+
+    assert describe([16384]) == (1, 256, 0)            # config 4's chunk on its own: 16 tiles, too few to permute
+    assert describe([65536]) == (1, 256, 1)            # 64 tiles
+    assert describe([2097152]) == (1, 256, 1)          # config 4's merged ring step
+    assert describe([2097152 + 1024]) == (1, 128, 1)   # 2049 tiles: 128-thread workgroups from here
+    assert describe([8388608]) == (1, 128, 1)          # config 2's ring step
+    assert describe([25165824, 25165824]) == (1, 128, 1)  # config 3's first halving step, two segments
+    assert describe([33554432]) == (1, 128, 1)
+    assert describe([33554432 + 1024]) == (1, 128, 0)  # beyond 32 Mi fp32 the plain order is the faster one
+    assert describe([67108864]) == (1, 128, 0)
+    assert describe([8388608], H.F64) == (1, 128, 1) and describe([1048576], H.F64) == (1, 256, 1)  # limits are in bytes
+    assert describe([4194303]) == (0, 256, 0)          # config 5's ragged last chunk: not a whole number of vectors
+    assert describe([8388608], base=(0x10000004, 0x20000004, 0x30000004)) == (0, 256, 0)  # off the 16-byte grid
+    assert describe([0, 8388608, 0]) == (1, 128, 1)    # empty segments do not count
+    assert describe([]) == (0, 256, 0)
+    assert L.ibcomm_hip_describe_launch(7, 0, None, None, None, None, None, None, None) == H.INVALID_ARGUMENT
