@@ -511,7 +511,7 @@ int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const 
 }
 
 int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, const void* const* a, const void* const* b,
-                               const size_t* len, int* aligned, int* threads, int* die_local) {
+                               const size_t* len, int* aligned, int* threads, int* die_local, int* write_through) {
   if (DTypeSize(dtype) == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
   if (n_segments < 0 || n_segments > kMaxSegments) return Fail(kInvalidArgument, "at most %d segments per launch", kMaxSegments);
   if (n_segments && (!dst || !a || !b || !len)) return Fail(kInvalidArgument, "null segment table");
@@ -523,6 +523,7 @@ int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, cons
   if (aligned) *aligned = shape.aligned ? 1 : 0;
   if (threads) *threads = shape.threads;
   if (die_local) *die_local = shape.die_local ? 1 : 0;
+  if (write_through) *write_through = shape.write_through ? 1 : 0;
   return kOk;
 }
 

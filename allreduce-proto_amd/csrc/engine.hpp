@@ -84,6 +84,7 @@ struct EngineStats {
   uint64_t reduce_kernel_segments = 0;  // segments the reduction launches carried after merging contiguous chunks
   uint64_t largest_reduce_elements = 0;  // the reduction launch with the most elements: its elements ...
   uint64_t largest_reduce_kernel_segments = 0;  // ... and its kernel segments
+  uint64_t largest_reduce_launches = 0;  // how many reduction launches had that many elements
 };
 
 template <class B>
@@ -616,8 +617,12 @@ class Communicator {
         outstanding_sends_--;
         if (c.has_done) NotePull(c.done, c.done_stream);
         if (s.dep >= 0 && staged_[s.dep] != nullptr) {
-          // the peer has fetched the staged partial sum: the slot is free once its read completes
+          // the peer has fetched the staged partial sum: the slot is free once its read completes.  A
+          // peer that reads nothing (a ghost in a replay) hands back no event; the slot's next user
+          // must then at least follow the launch that wrote it.
+          const OpState& wrote = recv_done_[s.dep];
           if (c.has_done) controller_.returnMemory(staged_[s.dep], c.done, c.done_stream);
+          else if (wrote.has_event) controller_.returnMemory(staged_[s.dep], wrote.event, wrote.stream);
           else controller_.returnMemory(staged_[s.dep]);
           staged_[s.dep] = nullptr;
         } else if (s.dep >= 0 || in_place_) {
@@ -895,7 +900,9 @@ class Communicator {
     if (launch_elements > stats_.largest_reduce_elements) {
       stats_.largest_reduce_elements = launch_elements;
       stats_.largest_reduce_kernel_segments = batch.count;
+      stats_.largest_reduce_launches = 0;
     }
+    if (launch_elements == stats_.largest_reduce_elements) stats_.largest_reduce_launches++;
     OpState done;
     IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
     trace_.Mark(Trace::kIssueReduKernel);

@@ -12,7 +12,9 @@
 //     *enqueued*, together with the event that marks that kernel's completion;
 //     the next user of the slot orders itself after that event on the device.
 //     The host never waits for a slot, so a handful of slots sustain the whole
-//     pipeline and the pool does not grow with the buffer;
+//     pipeline and the pool does not grow with the buffer; returned slots are
+//     reused before untouched ones, so those few slots are also all the memory
+//     a collective's staging ever writes;
 //   * each slot keeps 16 spare bytes so that a message can land at the same
 //     16-byte phase as the recvbuf range it will be added to, which keeps the
 //     kernel's body on dwordx4 accesses for odd chunk offsets;
@@ -65,7 +67,12 @@ class MemoryController {
   int held() const { return held_; }
   int high_water() const { return high_water_; }
 
-  // FIFO hand-out (memory_pool.h:222-236).  Grows the pool by one block if no slot is vacant.
+  // Hand-out (memory_pool.h:222-236): the slot that came back longest ago, else one that has never
+  // been used, else the pool grows by one block.  Preferring returned slots keeps the memory a
+  // collective writes to as small as its pipeline depth (a handful of slots) however large the
+  // block is; on MI355X that working set then lives in the 256 MB memory-side cache, and a ring
+  // step's stores into it run measurably faster than stores that walk through the whole block
+  // (config 2: 205 -> 196 us per rank schedule).
   int getMemory(Memory<B>** out);
   // FIFO return (memory_pool.h:238-242); `after` completes when the slot's contents are dead.
   void returnMemory(Memory<B>* m, typename B::Event after, typename B::Stream stream) {
@@ -89,7 +96,8 @@ class MemoryController {
   size_t stride_ = 0;
   bool descending_ = false;
   std::vector<std::unique_ptr<Memory<B>>> slots_;
-  std::deque<Memory<B>*> vacant_;
+  std::deque<Memory<B>*> vacant_;  // returned, oldest first
+  std::deque<Memory<B>*> fresh_;   // never handed out, in address order of the hand-out direction
   int held_ = 0;
   int high_water_ = 0;
 };
@@ -134,6 +142,7 @@ class MemoryPool {
     c->descending_ = descending;
     c->slots_.clear();
     c->vacant_.clear();
+    c->fresh_.clear();
     c->held_ = 0;
     c->high_water_ = 0;
     for (auto& b : blocks_) c->Carve(b.first, b.second);
@@ -242,22 +251,23 @@ void MemoryController<B>::Carve(char* block, size_t block_bytes) {
     Memory<B>* m = slots_.back().get();
     m->base = block + i * stride_;
     m->capacity = stride_;
-    vacant_.push_back(m);
+    fresh_.push_back(m);
   }
 }
 
 template <class B>
 int MemoryController<B>::getMemory(Memory<B>** out) {
   if (!pool_) return Fail(kInvalidArgument, "MemoryController is not attached to a pool");
-  if (vacant_.empty()) {
+  if (vacant_.empty() && fresh_.empty()) {
     size_t bytes = pool_->block_bytes();
     if (bytes < 2 * stride_) bytes = 2 * stride_;
     char* block = nullptr;
     IBCOMM_RETURN_IF_ERROR(pool_->AllocateBlock(bytes, &block));
     Carve(block, bytes);
   }
-  Memory<B>* m = vacant_.front();
-  vacant_.pop_front();
+  std::deque<Memory<B>*>& from = vacant_.empty() ? fresh_ : vacant_;
+  Memory<B>* m = from.front();
+  from.pop_front();
   held_++;
   if (held_ > high_water_) high_water_ = held_;
   *out = m;
@@ -269,6 +279,7 @@ void MemoryController<B>::Release() {
   if (!pool_) return;
   slots_.clear();
   vacant_.clear();
+  fresh_.clear();
   pool_->CompleteMemoryController();
   pool_ = nullptr;
 }

@@ -14,10 +14,13 @@ constexpr int kGeneralThreads = 256;
 // twice, so neither the L2 nor the memory-side cache should keep the lines.  Stores of the aligned
 // kernel carry the system coherence scope instead (sc1): they are written through to the memory
 // side, where the 256 MB cache in front of HBM absorbs them and writes them back in longer runs
-// than the kernel's own interleaving of two reads and one write would give the DRAM.  Measured on
-// MI355X against non-temporal stores: copies of 32 to 64 MiB 3 to 4 % faster, adds 1 to 3 %
-// faster up to 64 MiB per operand, no difference beyond.  The builtin offers no such store, hence
-// the one instruction of inline assembly; the compiler still schedules everything around it.
+// than the kernel's own interleaving of two reads and one write would give the DRAM; and a
+// destination that is written again soon (a rank's few staging slots) is still there.  Measured on
+// MI355X against non-temporal stores: a ring step of 32 MiB per operand into a 64 MiB staging ring
+// 7 % faster, copies of 32 to 64 MiB 3 to 4 % faster, nothing gained once a launch writes more
+// than about half that cache, where non-temporal stores are 1 to 2 % ahead; the host picks by the
+// bytes a launch writes.  The builtin offers no such store, hence the one instruction of inline
+// assembly; the compiler still schedules everything around it.
 template <typename V>
 __device__ __forceinline__ void StoreWriteThrough(V* p, V v) {
   static_assert(sizeof(V) == 16, "one 16-byte vector");
@@ -30,13 +33,15 @@ template <int N>
 struct KernelSegments {
   Segment seg[N];
   uint32_t die_local_tiles;
+  uint32_t write_through;  // stores carry the system scope (see StoreWriteThrough) instead of the non-temporal hint
 };
 
 template <int N>
-KernelSegments<N> MakeKernelSegments(const SegmentBatch& batch, uint32_t die_local_tiles) {
+KernelSegments<N> MakeKernelSegments(const SegmentBatch& batch, uint32_t die_local_tiles, uint32_t write_through) {
   KernelSegments<N> k;
   for (int i = 0; i < batch.count && i < N; i++) k.seg[i] = batch.seg[i];
   k.die_local_tiles = die_local_tiles;
+  k.write_through = write_through;
   return k;
 }
 
@@ -97,21 +102,22 @@ __global__ __launch_bounds__(kGeneralThreads) void SegmentKernel(const KernelSeg
 // consecutive tiles (32 KiB of each operand) of the group: a few percent faster for launches up to
 // some tens of megabytes per operand, slower beyond, so the host sets it by launch size (0 = plain).
 template <typename V, int THREADS, bool ADD>
-__device__ __forceinline__ void AlignedTile(V* dst, const V* a, const V* b, uint64_t nvec, uint32_t die_local_tiles) {
+__device__ __forceinline__ void AlignedTile(V* dst, const V* a, const V* b, uint64_t nvec, uint32_t die_local_tiles, uint32_t write_through) {
   uint64_t tile = blockIdx.x;
   if (tile < die_local_tiles) tile = (tile & ~63ull) + (tile % 8) * 8 + (tile / 8) % 8;
   const uint64_t i = tile * THREADS + threadIdx.x;
   if (i >= nvec) return;
   V v = __builtin_nontemporal_load(a + i);
   if (ADD) v = v + __builtin_nontemporal_load(b + i);
-  StoreWriteThrough(dst + i, v);
+  if (write_through) StoreWriteThrough(dst + i, v);
+  else __builtin_nontemporal_store(v, dst + i);
 }
 
 template <typename V, int PER_VEC, int THREADS, bool ADD>
 __global__ __launch_bounds__(THREADS) void AlignedSegmentKernel(const KernelSegments<kMaxSegments> batch) {
   const Segment s = batch.seg[blockIdx.y];
   AlignedTile<V, THREADS, ADD>(static_cast<V*>(s.dst), static_cast<const V*>(s.a), static_cast<const V*>(s.b), s.n / PER_VEC,
-                               batch.die_local_tiles);
+                               batch.die_local_tiles, batch.write_through);
 }
 
 // A launch of one segment (a ring step whose chunks merged into one) takes its operands as plain
@@ -119,29 +125,31 @@ __global__ __launch_bounds__(THREADS) void AlignedSegmentKernel(const KernelSegm
 // registers, where the table form costs every workgroup a scalar load from a 2 KiB argument block
 // before it can issue its only loads.
 template <typename V, int THREADS, bool ADD>
-__global__ __launch_bounds__(THREADS) void AlignedOneSegmentKernel(V* dst, const V* a, const V* b, uint64_t nvec, uint32_t die_local_tiles) {
-  AlignedTile<V, THREADS, ADD>(dst, a, b, nvec, die_local_tiles);
+__global__ __launch_bounds__(THREADS) void AlignedOneSegmentKernel(V* dst, const V* a, const V* b, uint64_t nvec, uint32_t die_local_tiles,
+                                                                   uint32_t write_through) {
+  AlignedTile<V, THREADS, ADD>(dst, a, b, nvec, die_local_tiles, write_through);
 }
 
 namespace {
 
 template <typename V, int PER_VEC, int THREADS>
-hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool add, bool die_local, hipStream_t stream) {
+hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream) {
   const uint64_t blocks = (max_nvec + THREADS - 1) / THREADS;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
-  const uint32_t die_local_tiles = die_local ? static_cast<uint32_t>(blocks & ~63ull) : 0u;
+  const uint32_t die_local_tiles = shape.die_local ? static_cast<uint32_t>(blocks & ~63ull) : 0u;
+  const uint32_t write_through = shape.write_through ? 1u : 0u;
   // A copy moves bits: the element types of one width share a copy kernel.
   if (batch.count == 1) {
     const Segment& s = batch.seg[0];
     if (add)
       hipLaunchKernelGGL((AlignedOneSegmentKernel<V, THREADS, true>), grid, dim3(THREADS), 0, stream, static_cast<V*>(s.dst),
-                         static_cast<const V*>(s.a), static_cast<const V*>(s.b), max_nvec, die_local_tiles);
+                         static_cast<const V*>(s.a), static_cast<const V*>(s.b), max_nvec, die_local_tiles, write_through);
     else
       hipLaunchKernelGGL((AlignedOneSegmentKernel<u32x4, THREADS, false>), grid, dim3(THREADS), 0, stream, static_cast<u32x4*>(s.dst),
-                         static_cast<const u32x4*>(s.a), static_cast<const u32x4*>(nullptr), max_nvec, die_local_tiles);
+                         static_cast<const u32x4*>(s.a), static_cast<const u32x4*>(nullptr), max_nvec, die_local_tiles, write_through);
   } else {
-    const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, die_local_tiles);
+    const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, die_local_tiles, write_through);
     if (add) hipLaunchKernelGGL((AlignedSegmentKernel<V, PER_VEC, THREADS, true>), grid, dim3(THREADS), 0, stream, args);
     else hipLaunchKernelGGL((AlignedSegmentKernel<u32x4, PER_VEC, THREADS, false>), grid, dim3(THREADS), 0, stream, args);
   }
@@ -150,13 +158,13 @@ hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool a
 
 template <typename V, int PER_VEC>
 hipError_t LaunchAligned(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream) {
-  return shape.threads == 256 ? LaunchAlignedOne<V, PER_VEC, 256>(batch, max_nvec, add, shape.die_local, stream)
-                              : LaunchAlignedOne<V, PER_VEC, 128>(batch, max_nvec, add, shape.die_local, stream);
+  return shape.threads == 256 ? LaunchAlignedOne<V, PER_VEC, 256>(batch, max_nvec, add, shape, stream)
+                              : LaunchAlignedOne<V, PER_VEC, 128>(batch, max_nvec, add, shape, stream);
 }
 
 template <typename T, typename V, typename CopyT, typename CopyV>
 hipError_t LaunchGeneral(const SegmentBatch& batch, dim3 grid, bool add, hipStream_t stream) {
-  const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, 0);
+  const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, 0, 0);
   if (add) hipLaunchKernelGGL((SegmentKernel<T, V, true>), grid, dim3(kGeneralThreads), 0, stream, args);
   else hipLaunchKernelGGL((SegmentKernel<CopyT, CopyV, false>), grid, dim3(kGeneralThreads), 0, stream, args);
   return hipGetLastError();
@@ -169,7 +177,7 @@ namespace {
 // Drops empty segments (their pointers may be anything), checks the rest and decides how the launch
 // is issued.  *max_n is the length of the longest segment; 0 means there is nothing to launch.
 hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, LaunchShape* shape, uint64_t* max_n) {
-  *shape = LaunchShape{false, kGeneralThreads, false, 0};
+  *shape = LaunchShape{false, kGeneralThreads, false, false, 0};
   *max_n = 0;
   batch->count = 0;
   if (given.count <= 0) return hipSuccess;
@@ -178,12 +186,14 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
   if (es == 0) return hipErrorInvalidValue;
   const uint64_t per_vec = 16 / es;
   uintptr_t misfit = 0;  // any low pointer bit, any length remainder
+  uint64_t written = 0;  // bytes the launch stores
   for (int i = 0; i < given.count; i++) {
     const Segment& s = given.seg[i];
     if (s.n == 0) continue;
     if (!s.dst || !s.a) return hipErrorInvalidValue;
     if (batch->count && (s.b != nullptr) != (batch->seg[0].b != nullptr)) return hipErrorInvalidValue;  // all adds or all copies
     if (s.n > *max_n) *max_n = s.n;
+    written += s.n * es;
     misfit |= ((reinterpret_cast<uintptr_t>(s.dst) | reinterpret_cast<uintptr_t>(s.a) | reinterpret_cast<uintptr_t>(s.b)) & 15) |
               (s.n % per_vec);
     batch->seg[batch->count++] = s;
@@ -201,6 +211,9 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
   shape->aligned = true;
   shape->threads = tiles >= kWg128MinTiles ? 128 : 256;
   shape->die_local = tiles >= 64 && tiles <= kDieLocalMaxTiles;
+  // Stores go through the memory-side cache while a launch writes at most half of its 256 MB
+  // (config 2's ring step writes 32 MiB, config 5's 64 MiB; config 3's first halving step 192 MiB).
+  shape->write_through = written <= (uint64_t(128) << 20);
   return hipSuccess;
 }
 

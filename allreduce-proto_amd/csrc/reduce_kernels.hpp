@@ -48,6 +48,7 @@ struct LaunchShape {
   bool aligned;    // AlignedSegmentKernel (true) or SegmentKernel (false)
   int threads;     // workgroup size: 256, or 128 for large aligned segments
   bool die_local;  // aligned kernel only: tiles ordered so that each die gets runs of 8 consecutive tiles
+  bool write_through;  // aligned kernel only: stores written through the memory-side cache instead of past it
   int segments;    // non-empty segments
 };
 

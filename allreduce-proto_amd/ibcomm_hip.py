@@ -39,7 +39,7 @@ class Stats(C.Structure):
         "calls", "reduce_launches", "reduce_segments", "reduce_elements", "landing_copies", "landing_bytes",
         "gather_copies", "gather_bytes", "messages_sent", "messages_received", "events_recorded", "stream_waits",
         "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes", "reduce_kernel_segments",
-        "largest_reduce_elements", "largest_reduce_kernel_segments")]
+        "largest_reduce_elements", "largest_reduce_kernel_segments", "largest_reduce_launches")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -74,7 +74,7 @@ def lib():
     L.ibcomm_hip_reduce.argtypes = [i, vp, vp, vp, sz, vp]
     L.ibcomm_hip_reduce_segments.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), vp]
     L.ibcomm_hip_copy_segments.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), vp]
-    L.ibcomm_hip_describe_launch.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), C.POINTER(i), C.POINTER(i), C.POINTER(i)]
+    L.ibcomm_hip_describe_launch.argtypes = [i, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), C.POINTER(i), C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_split_buffer.argtypes = [sz, sz, i, C.c_char_p, C.POINTER(sz), C.POINTER(sz), i, C.POINTER(i)]
     L.ibcomm_hip_rank_to_chunk.argtypes = [i, i, C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_get_exp_of_two.argtypes = [i]

@@ -113,12 +113,14 @@ def check_result(torch, O, H, algo, send, recv, chunk):
     return bool(ok)
 
 
-def launch_tables(send, recv, seg_elems, k):
-    """Operand tables for launches of k segments x seg_elems: every operand of every segment a distinct
-    range, successive launches walking through all ranks' buffers (several GiB), and no operand that is
-    read was written by an earlier launch, so nothing is served from a cache (a recently written operand
-    would be: stores that carry a coherence scope leave their lines in the 256 MB memory-side cache):
-    a and b come from two ranks' sendbufs at the same offset, dst from a recvbuf."""
+def launch_tables(send, recv, seg_elems, k, staging=None):
+    """Operand tables for launches of k segments x seg_elems.  The operands that are READ are distinct
+    ranges of two ranks' sendbufs at the same offset, successive launches walking through all ranks'
+    buffers (at least 2 GiB per pass), none of them ever written: nothing that is read comes out of a
+    cache.  The operand that is WRITTEN goes where the schedule puts it: with `staging` (a device
+    buffer of the size of a rank's staging working set) the launches cycle through that buffer, as a
+    rank's reductions cycle through the few pool slots they stage their results in; without it dst
+    walks through all ranks' recvbufs."""
     world = len(send)
     vp = C.c_void_p
     n = send[0].numel()
@@ -126,13 +128,17 @@ def launch_tables(send, recv, seg_elems, k):
     shapes = []
     # enough launches' worth of distinct operands that a pass over the tables reads at least 2 GiB
     tables = max(world * 2, -(-(2 << 30) // (8 * seg_elems * k)))
+    stage_segments = max(1, staging.numel() // seg_elems) if staging is not None else 0
     for i in range(tables):
         dst, a, b = [], [], []
         for j in range(k):
             idx = (i * k + j)
             r = idx % world
             off = ((idx // world) % per_buf) * seg_elems * 4
-            dst.append(recv[r].data_ptr() + off)
+            if staging is not None:
+                dst.append(staging.data_ptr() + (idx % stage_segments) * seg_elems * 4)
+            else:
+                dst.append(recv[r].data_ptr() + off)
             a.append(send[r].data_ptr() + off)
             b.append(send[(r + world // 2) % world].data_ptr() + off)
         shapes.append(((vp * k)(*dst), (vp * k)(*a), (vp * k)(*b), (C.c_size_t * k)(*([seg_elems] * k))))
@@ -154,11 +160,11 @@ def time_launches(torch, stream, launch, launches, warm=5):
     return e0.elapsed_time(e1) * 1e-3 / launches
 
 
-def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
+def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches, staging=None):
     """Average duration of the dominant kernel at its in-schedule launch shape, HIP events on its own stream."""
     stream = torch.cuda.Stream()
     k = segs_per_launch
-    shapes = launch_tables(send, recv, seg_elems, k)
+    shapes = launch_tables(send, recv, seg_elems, k, staging)
     L = H.lib()
 
     def launch(i):
@@ -168,9 +174,9 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
 
     avg_s = time_launches(torch, stream, launch, launches)
     algorithmic = 12.0 * seg_elems * k
-    aligned, threads, die_local = C.c_int(), C.c_int(), C.c_int()
+    aligned, threads, die_local, through = C.c_int(), C.c_int(), C.c_int(), C.c_int()
     d, a, b, ln = shapes[0]
-    assert L.ibcomm_hip_describe_launch(H.F32, k, d, a, b, ln, C.byref(aligned), C.byref(threads), C.byref(die_local)) == 0
+    assert L.ibcomm_hip_describe_launch(H.F32, k, d, a, b, ln, C.byref(aligned), C.byref(threads), C.byref(die_local), C.byref(through)) == 0
     shape = "%d segments x %d fp32" % (k, seg_elems)
     return {
         "bound": "hbm",
@@ -180,12 +186,15 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches):
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
         # counter traffic is known for the kernel geometry it was collected on, and only for that
         "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value)) if aligned.value else None,
-        "kernel": "ibcomm_hip::%s<float4, %d threads, add, %s tile order>" % (
-            "AlignedSegmentKernel" if aligned.value else "SegmentKernel", threads.value, "die-local" if die_local.value else "plain"),
+        "kernel": "ibcomm_hip::%s<float4, %d threads, add>, %s tile order, non-temporal loads, %s stores" % (
+            ("AlignedOneSegmentKernel" if k == 1 else "AlignedSegmentKernel") if aligned.value else "SegmentKernel", threads.value,
+            "die-local" if die_local.value else "plain", "written-through (sc1)" if through.value else "non-temporal"),
         "launch_shape": shape,
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
         "launches_timed": launches,
+        "result_goes_to": ("a staging region of %d bytes, cycled through as a rank's reductions cycle through their pool slots"
+                           % (staging.numel() * 4)) if staging is not None else "all ranks' recvbufs in turn",
     }
 
 
@@ -214,7 +223,7 @@ def bench_lib():
     return _bench_lib
 
 
-def variant_times(torch, H, send, recv, total_elems, add, launches=60, passes=3):
+def variant_times(torch, H, send, recv, total_elems, add, launches=60, passes=3, staging=None):
     """Every variant that takes `total_elems` fp32 in one segment, and the shipped kernel on the same
     operands: -> [(name, seconds per launch)], shipped kernel first.  Each figure is the median of
     `passes` HIP-event averages over `launches` back-to-back launches; the passes go round all variants,
@@ -223,7 +232,7 @@ def variant_times(torch, H, send, recv, total_elems, add, launches=60, passes=3)
     B = bench_lib()
     L = H.lib()
     stream = torch.cuda.Stream()
-    shapes = launch_tables(send, recv, total_elems, 1)
+    shapes = launch_tables(send, recv, total_elems, 1, staging)
 
     def shipped(i):
         d, a, b, ln = shapes[i % len(shapes)]
@@ -249,12 +258,12 @@ def variant_times(torch, H, send, recv, total_elems, add, launches=60, passes=3)
     return [(name, sorted(samples[k])[passes // 2]) for k, (name, _) in enumerate(runners)]
 
 
-def ceiling_leg(torch, H, send, recv, seg_elems, segs_per_launch, shipped_us, full=False):
+def ceiling_leg(torch, H, send, recv, seg_elems, segs_per_launch, shipped_us, full=False, staging=None):
     """How far the shipped kernel is from the best any measured form of the kernel reaches at this launch
     size ("the ceiling"), what the shipped kernel sustains once a launch is large, and the runtime's own
     device-to-device copy as a 1 read : 1 write datum."""
     total = seg_elems * segs_per_launch
-    times = variant_times(torch, H, send, recv, total, add=True)
+    times = variant_times(torch, H, send, recv, total, add=True, staging=staging)
     best = min(times[1:], key=lambda t: t[1])
     again = times[0][1]
     out = {
@@ -485,19 +494,32 @@ def main():
         # follow one another in all three operands share a kernel segment.
         leg_segments = max(1, st_rank["largest_reduce_kernel_segments"])
         seg_elems = st_rank["largest_reduce_elements"] // leg_segments
+        # Where that launch's result goes in the schedule: into the pool slots the rank stages partial sums in,
+        # a working set of `slots_high_water` chunks (taken from the full-world run).  If launches of the dominant
+        # shape follow one another within a call (every ring step), their results cycle through that working set,
+        # and the leg's results do the same.  If the shape occurs once per call (the first halving step), everything
+        # else the rank writes in a call lies between two of its launches, and the leg's results cycle through a
+        # region of that size instead: the distance after which a location is written again is what decides
+        # whether the 256 MB memory-side cache still holds it.
+        staging_elems = max(s["slots_high_water"] for s in st) * (chunk // 4)
+        written_per_call = st_rank["reduce_elements"] + st_rank["gather_bytes"] // 4 + st_rank["landing_bytes"] // 4
+        if st_rank["largest_reduce_launches"] < 2:
+            staging_elems = max(staging_elems, written_per_call)
+        staging = torch.empty(max(staging_elems, seg_elems * leg_segments), device="cuda")
 
         if args.sweep or args.ceiling or args.overlap:
             total = seg_elems * leg_segments
             if args.sweep:
                 print_variant_table("dst = a + b, %d fp32 in one segment (12 B per element)" % total,
-                                    variant_times(torch, H, send, recv, total, True), 12.0 * total)
+                                    variant_times(torch, H, send, recv, total, True, staging=staging), 12.0 * total)
                 print()
                 print_variant_table("dst = a (the gather and landing copies), %d fp32 in one segment (8 B per element)" % total,
                                     variant_times(torch, H, send, recv, total, False), 8.0 * total)
             if args.ceiling:
-                leg = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+                leg = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)
                 print(json.dumps({"config": args.config, "roofline": leg,
-                                  "ceiling": ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], full=True)}))
+                                  "ceiling": ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], full=True,
+                                                         staging=staging)}))
             if args.overlap:
                 overlap_leg(torch, send, recv, total)
             return
@@ -508,7 +530,7 @@ def main():
                 recv[0].copy_(send[0])
             torch.cuda.synchronize()
             print(json.dumps({"only_roofline": True, "config": args.config,
-                              "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)}))
+                              "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)}))
             return
         # the C entry point with its arguments converted once, as any caller in a loop would hold them
         replay_fn = H.lib().ibcomm_hip_replay_allreduce
@@ -609,8 +631,13 @@ def main():
         },
     }
     if not args.no_roofline:
-        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
-        line["roofline"]["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, line["roofline"]["avg_launch_us"])
+        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)
+        # the same launches with the result walking through all ranks' recvbufs instead (2 GiB and more): what
+        # the one reduction per schedule whose result stays in recvbuf sees
+        far = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+        line["roofline"]["result_walking_through_all_recvbufs"] = {k: far[k] for k in ("avg_launch_us", "achieved", "frac")}
+        line["roofline"]["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, line["roofline"]["avg_launch_us"],
+                                                  staging=staging)
         if args.whole_buffer:
             # the same kernel over one whole per-rank buffer: what it sustains once the launch is large.
             # Not part of the default run, so that a profile of the default run holds the dominant
@@ -618,7 +645,7 @@ def main():
             whole = roofline_leg(torch, H, send, recv, n, 1, 40)
             line["roofline"]["whole_buffer_launch"] = {k: whole[k] for k in (
                 "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
-    del recv
+    del recv, staging
     if not args.no_cpu:
         del send
         torch.cuda.empty_cache()

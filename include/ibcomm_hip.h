@@ -170,10 +170,11 @@ int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const 
                              const size_t* len_elements, void* stream);
 /* How ibcomm_hip_reduce_segments would issue these segments, without launching: *aligned = 1 for the
  * kernel that takes 16-byte aligned pointers and whole vectors (0: the general kernel), *threads the
- * workgroup size, *die_local = 1 if tiles are ordered in runs per accelerator die.  Stands for the
- * launch geometry the reference fixes at ibcomm/allreduce_cuda_impl.h:24, 116-117. */
+ * workgroup size, *die_local = 1 if tiles are ordered in runs per accelerator die, *write_through = 1
+ * if the stores go through the memory-side cache (0: non-temporal).  Stands for the launch geometry
+ * the reference fixes at ibcomm/allreduce_cuda_impl.h:24, 116-117. */
 int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, const void* const* a, const void* const* b,
-                               const size_t* len_elements, int* aligned, int* threads, int* die_local);
+                               const size_t* len_elements, int* aligned, int* threads, int* die_local, int* write_through);
 
 /* ---- point-to-point messaging over the loopback ------------------------------------------------ */
 
@@ -261,6 +262,7 @@ typedef struct {
                                       another in all three operands are merged into one segment */
   uint64_t largest_reduce_elements;        /* the reduction launch with the most elements: its elements */
   uint64_t largest_reduce_kernel_segments; /* ... and its kernel segments */
+  uint64_t largest_reduce_launches;        /* how many reduction launches had that many elements */
 } ibcomm_hip_stats;
 
 int ibcomm_hip_comm_stats(ibcomm_hip_comm* comm, ibcomm_hip_stats* out);

@@ -19,7 +19,7 @@ class EngineStats(C.Structure):
         "calls", "reduce_launches", "reduce_segments", "reduce_elements", "landing_copies", "landing_bytes",
         "gather_copies", "gather_bytes", "messages_sent", "messages_received", "events_recorded", "stream_waits",
         "streams_created", "slots_high_water", "slot_count", "pool_blocks", "pool_bytes", "progress_passes", "reduce_kernel_segments",
-        "largest_reduce_elements", "largest_reduce_kernel_segments")]
+        "largest_reduce_elements", "largest_reduce_kernel_segments", "largest_reduce_launches")]
 
 
 class Report(C.Structure):

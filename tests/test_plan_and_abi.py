@@ -141,9 +141,12 @@ def test_launch_geometry_follows_the_segment_size():
         a = (vp * k)(*[base[1] + i * 0x1000000 for i in range(k)])
         b = (vp * k)(*[base[2] + i * 0x1000000 for i in range(k)])
         ln = (C.c_size_t * k)(*lens)
-        al, th, dl = C.c_int(-1), C.c_int(-1), C.c_int(-1)
-        assert L.ibcomm_hip_describe_launch(dtype, k, d, a, b, ln, C.byref(al), C.byref(th), C.byref(dl)) == 0, H.last_error()
+        al, th, dl, wt = C.c_int(-1), C.c_int(-1), C.c_int(-1), C.c_int(-1)
+        assert L.ibcomm_hip_describe_launch(dtype, k, d, a, b, ln, C.byref(al), C.byref(th), C.byref(dl), C.byref(wt)) == 0, H.last_error()
+        through.append(wt.value)
         return al.value, th.value, dl.value
+
+    through = []
 
     assert describe([16384]) == (1, 256, 0)            # config 4's chunk on its own: 16 tiles, too few to permute
     assert describe([65536]) == (1, 256, 1)            # 64 tiles
@@ -159,4 +162,9 @@ def test_launch_geometry_follows_the_segment_size():
     assert describe([8388608], base=(0x10000004, 0x20000004, 0x30000004)) == (0, 256, 0)  # off the 16-byte grid
     assert describe([0, 8388608, 0]) == (1, 128, 1)    # empty segments do not count
     assert describe([]) == (0, 256, 0)
-    assert L.ibcomm_hip_describe_launch(7, 0, None, None, None, None, None, None, None) == H.INVALID_ARGUMENT
+    assert L.ibcomm_hip_describe_launch(7, 0, None, None, None, None, None, None, None, None) == H.INVALID_ARGUMENT
+    # stores go through the memory-side cache while a launch writes at most 128 MiB
+    through.clear()
+    for lens in ([8388608], [16777216], [33554432], [33554432 + 4], [25165824, 25165824], [4194304] * 8, [4194304] * 9):
+        describe(lens)
+    assert through == [1, 1, 1, 0, 0, 1, 0]
