@@ -7,6 +7,7 @@
     python bench.py --sweep [--config N]              every kernel variant of the measurement library at the launch shape
     python bench.py --ceiling [--config N]            the best variant, the shipped kernel on a large launch, hipMemcpyAsync
     python bench.py --overlap [--config N]            other ways to issue a schedule of dependent launches, and to wait for it
+    python bench.py --call-breakdown [--config N]     where the time of one blocking call goes, from the library's own trace
 
 One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
 collective: every partial sum the rank receives is added to its own contribution (the result going
@@ -46,11 +47,12 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # each calibrated against a device copy of known size; the summaries with the commands are under
 # profiles/.  Shapes that have not been measured report null.
 MEASURED_TRAFFIC_BYTES = {
-    # (launch shape, workgroup size, die-local tile order) of the aligned kernel -> bytes
-    ("1 segments x 8388608 fp32", 128, 1): 100681210,     # config 2, profiles/segment_kernel_add_ring8_256MiB.md
-    ("2 segments x 25165824 fp32", 128, 1): 603978883,    # config 3, profiles/segment_kernel_add_traffic_rabenseifner16_ring8_64KiB_ring32_2GiB.md
-    ("1 segments x 2097152 fp32", 256, 1): 25180425,      # config 4, same file
-    ("1 segments x 16777216 fp32", 128, 1): 201346522,    # config 5, same file
+    # (launch shape, workgroup size, die-local tile order, written-through stores) of the aligned kernel -> bytes;
+    # all four from profiles/aligned_add_kernel_traffic_four_configs.md
+    ("1 segments x 8388608 fp32", 128, 1, 1): 100676300,     # config 2
+    ("2 segments x 25165824 fp32", 128, 1, 0): 603980781,    # config 3
+    ("1 segments x 2097152 fp32", 256, 1, 1): 25179438,      # config 4
+    ("1 segments x 16777216 fp32", 128, 1, 1): 201344831,    # config 5
 }
 
 CONFIGS = {
@@ -185,7 +187,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches, sta
         "unit": "GB/s",
         "frac": round(algorithmic / avg_s * 1e-9 / HBM_PEAK_GBPS, 4),
         # counter traffic is known for the kernel geometry it was collected on, and only for that
-        "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value)) if aligned.value else None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value, through.value)) if aligned.value else None,
         "kernel": "ibcomm_hip::%s<float4, %d threads, add>, %s tile order, non-temporal loads, %s stores" % (
             ("AlignedOneSegmentKernel" if k == 1 else "AlignedSegmentKernel") if aligned.value else "SegmentKernel", threads.value,
             "die-local" if die_local.value else "plain", "written-through (sc1)" if through.value else "non-temporal"),
@@ -407,6 +409,58 @@ def overlap_leg(torch, send, recv, seg_elems):
         print("    %-100s %8.2f us per call, %6.2f over device pace" % (name, t, t - base), flush=True)
 
 
+def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
+    """Where one blocking call of the rank's schedule spends its time, from the library's trace: per-launch device
+    durations when the call is issued eagerly, and for graph replays the host spans "graph launched" and "waiting for
+    the completion flag" next to the device's first-kernel-to-end duration."""
+    import statistics as st
+    import tempfile
+    fn = H.lib().ibcomm_hip_replay_allreduce
+    args = (w.comms[rank], C.c_int(algo), C.c_int(H.F32), C.c_void_p(send_ptr), C.c_void_p(out_ptr), C.c_size_t(n))
+
+    def wall(calls):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            assert fn(*args) == 0, H.last_error()
+        return (time.perf_counter() - t0) / calls * 1e6
+
+    def traced(calls):
+        base = os.path.join(tempfile.mkdtemp(), "trace")
+        os.environ["IBCOMM_TRACE_FILE"] = base
+        w.set_trace(True)
+        t = wall(calls)
+        w.dump_trace()
+        w.set_trace(False)
+        lines = {ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in open("%s_%d.dat" % (base, rank)).read().splitlines()}
+        return t, lines
+
+    for _ in range(5):
+        assert fn(*args) == 0, H.last_error()
+    print("graph replay, trace off: %8.2f us per call (host wall clock, 50 calls)" % wall(50))
+    t, lines = traced(50)
+    spans = list(zip(lines["other"][0::2], lines["other"][1::2]))
+    launch, wait = spans[0::2], spans[1::2]
+    print("graph replay, trace on:  %8.2f us per call; per call, medians of %d replays:" % (t, len(lines["device-graph"]) // 2))
+    print("    host, inside hipGraphLaunch (with the two timing events the trace adds)  %8.2f us" % (st.median(d for _, d in launch) * 1e3))
+    print("    host, spinning on the completion flag                                    %8.2f us" % (st.median(d for _, d in wait) * 1e3))
+    print("    device, event before the graph to event after it                         %8.2f us" % (st.median(lines["device-graph"][1::2]) * 1e3))
+    w.set_graph_mode(0)
+    for _ in range(3):
+        assert fn(*args) == 0, H.last_error()
+    print("eager issue, trace off:  %8.2f us per call" % wall(30))
+    t, lines = traced(30)
+    red, cp = lines["device-redu-kernel"][1::2], lines["device-copy-kernel"][1::2]
+    per_call_red, per_call_cp = len(red) // 30, len(cp) // 30
+    print("eager issue, trace on:   %8.2f us per call; device durations between the HIP events around each launch:" % t)
+    print("    %d reduction launches per call: median %.2f us, sum per call %.2f us" % (per_call_red, st.median(red) * 1e3, sum(red) / 30 * 1e3))
+    print("    %d copy launches per call:      median %.2f us, sum per call %.2f us" % (per_call_cp, st.median(cp) * 1e3, sum(cp) / 30 * 1e3))
+    issue = [lines[k][1::2] for k in ("issue-redu-kernel", "issue-copy-kernel", "issue-send", "received", "issue-recv", "reduced", "other")]
+    print("    host time per call in the trace's categories (us): issue-redu-kernel %.1f, issue-copy-kernel %.1f, issue-send %.1f, "
+          "received %.1f, issue-recv %.1f, reduced %.1f, other %.1f" % tuple(sum(v) / 30 * 1e3 for v in issue))
+    w.set_graph_mode(1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -420,6 +474,9 @@ def main():
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
+    ap.add_argument("--leg-shape", default=None, metavar="SEGMENTS,ELEMENTS,STAGING_ELEMENTS",
+                    help="with --only-roofline: time exactly this launch shape (as printed by a plain --only-roofline run as "
+                         "`leg_shape`) without running the collective first, so that a profile of the command holds the leg's launches only")
     ap.add_argument("--whole-buffer", action="store_true",
                     help="also time the reduction kernel over one whole per-rank buffer in a single segment "
                          "(roofline.whole_buffer_launch): what it sustains once a launch is large")
@@ -427,6 +484,9 @@ def main():
                     help="time every kernel variant of the measurement library, adds and copies, at the workload's launch shape")
     ap.add_argument("--ceiling", action="store_true",
                     help="the best variant at the launch shape, the shipped kernel on a whole-buffer launch, and hipMemcpyAsync")
+    ap.add_argument("--call-breakdown", action="store_true",
+                    help="run the rank's schedule with the library's trace on, eagerly and as graph replays, and print host spans "
+                         "and device durations per call")
     ap.add_argument("--overlap", action="store_true",
                     help="other ways of issuing the schedule's dependent launches (graph chains, streams, no-barrier launches, "
                          "ready counters) and of waiting for them")
@@ -466,6 +526,16 @@ def main():
             assert rc == 0, H.last_error()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
+
+    if args.only_roofline and args.leg_shape:
+        k, elems, staging_elems = (int(x) for x in args.leg_shape.split(","))
+        staging = torch.empty(max(staging_elems, k * elems), device="cuda")
+        for _ in range(3):  # the copies of known size that calibrate hardware counters (see below)
+            recv[0].copy_(send[0])
+        torch.cuda.synchronize()
+        print(json.dumps({"only_roofline": True, "config": args.config, "leg_shape": args.leg_shape,
+                          "roofline": roofline_leg(torch, H, send, recv, elems, k, 200, staging)}))
+        return
 
     rank = 0
     with H.World(world) as w:
@@ -507,6 +577,9 @@ def main():
             staging_elems = max(staging_elems, written_per_call)
         staging = torch.empty(max(staging_elems, seg_elems * leg_segments), device="cuda")
 
+        if args.call_breakdown:
+            call_breakdown(torch, H, w, rank, algo, sp[rank], out.data_ptr(), n)
+            return
         if args.sweep or args.ceiling or args.overlap:
             total = seg_elems * leg_segments
             if args.sweep:
@@ -530,6 +603,7 @@ def main():
                 recv[0].copy_(send[0])
             torch.cuda.synchronize()
             print(json.dumps({"only_roofline": True, "config": args.config,
+                              "leg_shape": "%d,%d,%d" % (leg_segments, seg_elems, staging.numel()),
                               "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)}))
             return
         # the C entry point with its arguments converted once, as any caller in a loop would hold them
