@@ -299,6 +299,9 @@ __global__ __launch_bounds__(T) void Flagged(f32x4* __restrict__ d, const f32x4*
 
 __global__ void SetFlag(volatile uint32_t* flag, uint32_t v) { *flag = v; }
 __global__ void Null() {}
+__global__ void StoreClock(uint64_t* host_word) {
+  __hip_atomic_store(host_word, static_cast<uint64_t>(wall_clock64()), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 struct Region {
   char *a, *b, *d;
@@ -524,6 +527,8 @@ int ibv_probe_flags(int flags, int any_order, void* ra, void* rb, void* rd, size
 //   method 2  eager launches + a one-thread kernel that writes a flag in pinned host memory; the host spins on the flag
 //   method 3  graph (one chain) + hipStreamSynchronize
 //   method 4  graph + the flag kernel (launched eagerly behind it) + host spins on the flag
+//   method 7  graph + hipStreamWriteValue64 of a flag in pinned host memory (a command-processor write, no kernel) + host spins
+//   method 9  graph whose last node stores the device clock to pinned host memory; host spins until the word changes (what the library does)
 //   method 5  `steps` empty kernels + hipStreamSynchronize (n ignored)
 //   method 6  `steps` empty kernels, calls back to back without waiting (the device's cost of a kernel boundary)
 int ibv_probe_blocking_call(int method, void* ra, void* rb, void* rd, size_t region_bytes, size_t n, int steps, int iters, double* us) {
@@ -537,7 +542,7 @@ int ibv_probe_blocking_call(int method, void* ra, void* rb, void* rd, size_t reg
   IBV_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   uint32_t* hflag = nullptr;
   IBV_CHECK(hipHostMalloc((void**)&hflag, 64, hipHostMallocMapped));
-  *hflag = 0;
+  hflag[0] = hflag[1] = 0;
   uint32_t* dflag = nullptr;
   IBV_CHECK(hipHostGetDevicePointer((void**)&dflag, hflag, 0));
   auto issue = [&]() {
@@ -556,7 +561,9 @@ int ibv_probe_blocking_call(int method, void* ra, void* rb, void* rd, size_t reg
   };
   std::vector<Args> args(steps);
   std::vector<void*> ptrs(static_cast<size_t>(steps) * 4);
-  if (method == 3 || method == 4) {
+  uint64_t* dclock = reinterpret_cast<uint64_t*>(dflag);
+  void* clock_args[1] = {&dclock};
+  if (method == 3 || method == 4 || method >= 7) {
     IBV_CHECK(hipGraphCreate(&g, 0));
     hipGraphNode_t last = nullptr;
     const bool small = n / 4 / 256 < 2049;
@@ -575,8 +582,19 @@ int ibv_probe_blocking_call(int method, void* ra, void* rb, void* rd, size_t reg
       IBV_CHECK(hipGraphAddKernelNode(&node, g, last ? &last : nullptr, last ? 1 : 0, &p));
       last = node;
     }
+    if (method == 9) {
+      hipKernelNodeParams p;
+      memset(&p, 0, sizeof p);
+      p.func = (void*)StoreClock;
+      p.gridDim = dim3(1);
+      p.blockDim = dim3(1);
+      p.kernelParams = clock_args;
+      hipGraphNode_t node;
+      IBV_CHECK(hipGraphAddKernelNode(&node, g, last ? &last : nullptr, last ? 1 : 0, &p));
+    }
     IBV_CHECK(hipGraphInstantiate(&ex, g, nullptr, nullptr, 0));
   }
+  const volatile uint64_t* hclock = reinterpret_cast<volatile uint64_t*>(hflag);
   uint32_t tick = 0;
   int rc = 0;
   switch (method) {
@@ -595,6 +613,19 @@ int ibv_probe_blocking_call(int method, void* ra, void* rb, void* rd, size_t reg
         tick++;
         hipLaunchKernelGGL(SetFlag, dim3(1), dim3(1), 0, s, (volatile uint32_t*)dflag, tick);
         while (*(volatile uint32_t*)hflag != tick) {}
+        return 0;
+      }, us); break;
+    case 7: rc = WallClock(3, iters, [&](int) {
+        IBV_CHECK(hipGraphLaunch(ex, s));
+        tick++;
+        IBV_CHECK(hipStreamWriteValue64(s, dflag, tick, 0));
+        while (*(volatile uint64_t*)hflag != tick) {}
+        return 0;
+      }, us); break;
+    case 9: rc = WallClock(3, iters, [&](int) {
+        const uint64_t before = *hclock;
+        IBV_CHECK(hipGraphLaunch(ex, s));
+        while (*hclock == before) {}
         return 0;
       }, us); break;
     case 5: rc = WallClock(3, iters, [&](int) {

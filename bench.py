@@ -404,7 +404,9 @@ def overlap_leg(torch, send, recv, seg_elems):
     print("one blocking call = issue the %d steps and return when they are done; host wall time per call, minus the device pace above (%.2f us):" % (steps, base))
     for method, name in ((0, "launches + hipStreamSynchronize"), (1, "launches + spin on hipStreamQuery"),
                          (2, "launches + a one-thread kernel writing a flag in pinned host memory, host spins on the flag"),
-                         (3, "graph replay + hipStreamSynchronize"), (4, "graph replay + the flag kernel, host spins on the flag")):
+                         (3, "graph replay + hipStreamSynchronize"), (4, "graph replay, then the flag kernel launched behind it, host spins on the flag"),
+                         (9, "graph whose last node stores the device clock to pinned host memory, host spins (what the library does)"),
+                         (7, "graph replay + hipStreamWriteValue64 of the flag (no kernel), host spins on the flag")):
         t = blocking(method)
         print("    %-100s %8.2f us per call, %6.2f over device pace" % (name, t, t - base), flush=True)
 
