@@ -373,11 +373,12 @@ int ibv_variant_launch(int v, void* dst, const void* a, const void* b, size_t n,
 //   mode 1  one stream, launches without the implicit barrier between them (hipExtAnyOrderLaunch)
 //   mode 2  an explicit HIP graph of kernel nodes: `chains` parallel chains, each taking 1/chains of every step
 //   mode 3  `chains` streams, issued eagerly, each taking 1/chains of every step
+//   mode 4  one stream, only every `chains`-th launch keeps the implicit barrier
 // Result: microseconds per schedule at device pace (schedules issued back to back, no host wait between).
 int ibv_probe_chains(int mode, void* ra, void* rb, void* rd, size_t region_bytes, size_t n, int steps, int chains, int iters, double* us) {
   const Region m = {static_cast<char*>(ra), static_cast<char*>(rb), static_cast<char*>(rd), region_bytes};
   const size_t bytes = n * 4, positions = m.bytes / bytes;
-  if (positions == 0 || chains < 1 || n % (static_cast<size_t>(chains) * 4 * 1024)) {
+  if (positions == 0 || chains < 1 || n % (static_cast<size_t>(mode == 4 ? 1 : chains) * 4 * 1024)) {
     snprintf(g_error, sizeof g_error, "bad shape");
     return 1;
   }
@@ -385,11 +386,13 @@ int ibv_probe_chains(int mode, void* ra, void* rb, void* rd, size_t region_bytes
   IBV_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   const uint64_t sub = n / chains, subvec = sub / 4;
   int rc = 0;
-  if (mode == 0 || mode == 1) {
+  if (mode == 0 || mode == 1 || mode == 4) {
+    // mode 4: every `chains`-th launch keeps the barrier, the others go without it
     rc = DevicePace(s, 2, iters, [&](int) {
       for (int r = 0; r < steps; r++) {
         const size_t pos = r % positions;
-        LaunchLikeShipped((f32x4*)(m.d + pos * bytes), (const f32x4*)(m.a + pos * bytes), (const f32x4*)(m.b + pos * bytes), n / 4, s, mode);
+        const unsigned flags = mode == 4 ? (r % chains == 0 ? 0u : 1u) : static_cast<unsigned>(mode);
+        LaunchLikeShipped((f32x4*)(m.d + pos * bytes), (const f32x4*)(m.a + pos * bytes), (const f32x4*)(m.b + pos * bytes), n / 4, s, flags);
       }
       return 0;
     }, us);

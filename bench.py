@@ -388,6 +388,7 @@ def overlap_leg(torch, send, recv, seg_elems):
 
     row("one stream, in-order launches (what the engine issues; a recorded graph is one such chain)", base)
     row("one stream, launches without the implicit barrier (hipExtAnyOrderLaunch; ignores the dependency)", chains(1, 1))
+    row("one stream, every 2nd launch without the implicit barrier (steps two apart still ordered)", chains(4, 2))
     for k in (1, 2, 4, 8):
         row("HIP graph of kernel nodes, %d parallel chain(s), each 1/%d of every step" % (k, k), chains(2, k))
     for k in (2, 4):
