@@ -126,7 +126,7 @@ int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, in
  * device work of all world_size ranks is enqueued on that one stream and the call returns without
  * waiting for it.  Staging slots come out of a 64 MiB array that is part of the library's code
  * object (one copy per GPU, held until the process ends): a call whose ranks could need more, i.e.
- * world_size * 2 * (chunks per buffer) * (chunk bytes rounded up to 256) > 64 MiB, returns 1 with a
+ * world_size * 2 * (chunks per buffer) * (chunk bytes + 16, rounded up to 256) > 64 MiB, returns 1 with a
  * message and enqueues nothing.  Calls on one GPU share the array: they must not overlap in time
  * (enqueue them on one stream, or synchronise in between).  The first call on a device looks up the
  * array's address and should be made outside a capture. */
