@@ -8,8 +8,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kGeneralThreads = 256;
-
 // Cache policy of the streaming accesses.  Loads carry the non-temporal hint: nothing is read
 // twice, so neither the L2 nor the memory-side cache should keep the lines.  Stores of the aligned
 // kernel carry the system coherence scope instead (sc1): they are written through to the memory
@@ -45,19 +43,21 @@ KernelSegments<N> MakeKernelSegments(const SegmentBatch& batch, uint32_t die_loc
   return k;
 }
 
-// One workgroup column (blockIdx.y) per segment; blockIdx.x is the tile of kGeneralThreads 16-byte
-// vectors.  T is the element type, V the 16-byte vector of T.  Integer types are instantiated
-// unsigned so that += wraps.  ADD selects dst = a + b; otherwise the launch is a copy, dst = a.
-// The two are separate kernels so that a profile tells reductions from landing copies.
-template <typename T, typename V, bool ADD>
-__global__ __launch_bounds__(kGeneralThreads) void SegmentKernel(const KernelSegments<kMaxSegments> batch) {
-  const Segment s = batch.seg[blockIdx.y];
-  const uint64_t n = s.n;
+// The die-local tile order (see AlignedTile below): within the first die_local_tiles tiles every
+// aligned group of 64 workgroup ids is transposed 8 x 8.
+__device__ __forceinline__ uint64_t TileOf(uint32_t block, uint32_t die_local_tiles) {
+  uint64_t tile = block;
+  if (tile < die_local_tiles) tile = (tile & ~63ull) + (tile % 8) * 8 + (tile / 8) % 8;
+  return tile;
+}
 
-  T* dst = static_cast<T*>(s.dst);
-  const T* a = static_cast<const T*>(s.a);
-  const T* b = static_cast<const T*>(s.b);
-
+// Any alignment, any length.  T is the element type, V the 16-byte vector of T.  Integer types
+// are instantiated unsigned so that += wraps.  ADD selects dst = a + b; otherwise the launch is a
+// copy, dst = a.  A segment whose pointers share their 16-byte phase is peeled: up to 16 bytes
+// element by element at each end, 16-byte vectors in between, with the tile order and the store
+// policy of the aligned kernel; any other segment goes element by element throughout.
+template <typename T, typename V, int THREADS, bool ADD>
+__device__ __forceinline__ void PeeledTile(T* dst, const T* a, const T* b, uint64_t n, uint32_t die_local_tiles, uint32_t write_through) {
   constexpr uint64_t kPerVec = 16 / sizeof(T);
   const uintptr_t pd = reinterpret_cast<uintptr_t>(dst) & 15;
   const bool same_phase = ((reinterpret_cast<uintptr_t>(a) & 15) == pd) &&
@@ -71,24 +71,41 @@ __global__ __launch_bounds__(kGeneralThreads) void SegmentKernel(const KernelSeg
     nvec = (n - head) / kPerVec;
   }
 
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * kGeneralThreads + threadIdx.x;
+  const uint64_t i = TileOf(blockIdx.x, die_local_tiles) * THREADS + threadIdx.x;
   if (i < nvec) {
     V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(a + head) + i);
     if (ADD) v = v + __builtin_nontemporal_load(reinterpret_cast<const V*>(b + head) + i);
-    __builtin_nontemporal_store(v, reinterpret_cast<V*>(dst + head) + i);
+    if (write_through) StoreWriteThrough(reinterpret_cast<V*>(dst + head) + i, v);
+    else __builtin_nontemporal_store(v, reinterpret_cast<V*>(dst + head) + i);
   }
 
   // Scalar remainder: fewer than two vectors' worth when the phases agree,
   // the whole segment when they do not.
   const uint64_t tail_begin = head + nvec * kPerVec;
   const uint64_t scalar_count = head + (n - tail_begin);
-  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kGeneralThreads;
-  for (uint64_t k = i; k < scalar_count; k += stride) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * THREADS;
+  for (uint64_t k = static_cast<uint64_t>(blockIdx.x) * THREADS + threadIdx.x; k < scalar_count; k += stride) {
     const uint64_t e = (k < head) ? k : tail_begin + (k - head);
     T v = a[e];
     if (ADD) v = v + b[e];
     dst[e] = v;
   }
+}
+
+// One workgroup column (blockIdx.y) per segment; blockIdx.x is the tile of THREADS 16-byte vectors.
+// Adds and copies are separate kernels so that a profile tells reductions from landing copies.
+template <typename T, typename V, int THREADS, bool ADD>
+__global__ __launch_bounds__(THREADS) void SegmentKernel(const KernelSegments<kMaxSegments> batch) {
+  const Segment s = batch.seg[blockIdx.y];
+  PeeledTile<T, V, THREADS, ADD>(static_cast<T*>(s.dst), static_cast<const T*>(s.a), static_cast<const T*>(s.b), s.n, batch.die_local_tiles,
+                                 batch.write_through);
+}
+
+// The same for a launch of one segment, operands as plain kernel arguments (see AlignedOneSegmentKernel).
+template <typename T, typename V, int THREADS, bool ADD>
+__global__ __launch_bounds__(THREADS) void OneSegmentKernel(T* dst, const T* a, const T* b, uint64_t n, uint32_t die_local_tiles,
+                                                            uint32_t write_through) {
+  PeeledTile<T, V, THREADS, ADD>(dst, a, b, n, die_local_tiles, write_through);
 }
 
 // The common case on its own: every pointer of every segment on a 16-byte boundary, every length a
@@ -103,9 +120,7 @@ __global__ __launch_bounds__(kGeneralThreads) void SegmentKernel(const KernelSeg
 // some tens of megabytes per operand, slower beyond, so the host sets it by launch size (0 = plain).
 template <typename V, int THREADS, bool ADD>
 __device__ __forceinline__ void AlignedTile(V* dst, const V* a, const V* b, uint64_t nvec, uint32_t die_local_tiles, uint32_t write_through) {
-  uint64_t tile = blockIdx.x;
-  if (tile < die_local_tiles) tile = (tile & ~63ull) + (tile % 8) * 8 + (tile / 8) % 8;
-  const uint64_t i = tile * THREADS + threadIdx.x;
+  const uint64_t i = TileOf(blockIdx.x, die_local_tiles) * THREADS + threadIdx.x;
   if (i >= nvec) return;
   V v = __builtin_nontemporal_load(a + i);
   if (ADD) v = v + __builtin_nontemporal_load(b + i);
@@ -162,12 +177,31 @@ hipError_t LaunchAligned(const SegmentBatch& batch, uint64_t max_nvec, bool add,
                               : LaunchAlignedOne<V, PER_VEC, 128>(batch, max_nvec, add, shape, stream);
 }
 
-template <typename T, typename V, typename CopyT, typename CopyV>
-hipError_t LaunchGeneral(const SegmentBatch& batch, dim3 grid, bool add, hipStream_t stream) {
-  const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, 0, 0);
-  if (add) hipLaunchKernelGGL((SegmentKernel<T, V, true>), grid, dim3(kGeneralThreads), 0, stream, args);
-  else hipLaunchKernelGGL((SegmentKernel<CopyT, CopyV, false>), grid, dim3(kGeneralThreads), 0, stream, args);
+template <typename T, typename V, int THREADS, bool ADD>
+hipError_t LaunchPeeledOne(const SegmentBatch& batch, uint64_t max_n, const LaunchShape& shape, hipStream_t stream) {
+  uint64_t blocks = (max_n / (16 / sizeof(T)) + THREADS - 1) / THREADS;
+  if (blocks == 0) blocks = 1;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
+  const uint32_t die_local_tiles = shape.die_local ? static_cast<uint32_t>(blocks & ~63ull) : 0u;
+  const uint32_t write_through = shape.write_through ? 1u : 0u;
+  if (batch.count == 1) {
+    const Segment& s = batch.seg[0];
+    hipLaunchKernelGGL((OneSegmentKernel<T, V, THREADS, ADD>), grid, dim3(THREADS), 0, stream, static_cast<T*>(s.dst), static_cast<const T*>(s.a),
+                       static_cast<const T*>(s.b), s.n, die_local_tiles, write_through);
+  } else {
+    const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, die_local_tiles, write_through);
+    hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, ADD>), grid, dim3(THREADS), 0, stream, args);
+  }
   return hipGetLastError();
+}
+
+// A copy moves bits: the element types of one width share a copy kernel (CopyT, CopyV).
+template <typename T, typename V, typename CopyT, typename CopyV>
+hipError_t LaunchPeeled(const SegmentBatch& batch, uint64_t max_n, bool add, const LaunchShape& shape, hipStream_t stream) {
+  if (shape.threads == 256)
+    return add ? LaunchPeeledOne<T, V, 256, true>(batch, max_n, shape, stream) : LaunchPeeledOne<CopyT, CopyV, 256, false>(batch, max_n, shape, stream);
+  return add ? LaunchPeeledOne<T, V, 128, true>(batch, max_n, shape, stream) : LaunchPeeledOne<CopyT, CopyV, 128, false>(batch, max_n, shape, stream);
 }
 
 }  // namespace
@@ -177,7 +211,7 @@ namespace {
 // Drops empty segments (their pointers may be anything), checks the rest and decides how the launch
 // is issued.  *max_n is the length of the longest segment; 0 means there is nothing to launch.
 hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, LaunchShape* shape, uint64_t* max_n) {
-  *shape = LaunchShape{false, kGeneralThreads, false, false, 0};
+  *shape = LaunchShape{false, 256, false, false, 0};
   *max_n = 0;
   batch->count = 0;
   if (given.count <= 0) return hipSuccess;
@@ -199,7 +233,7 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
     batch->seg[batch->count++] = s;
   }
   shape->segments = batch->count;
-  if (*max_n == 0 || misfit != 0) return hipSuccess;
+  if (*max_n == 0) return hipSuccess;
   // Measured on MI355X with fp32 (us per launch of one segment, 256 threads plain / 256 die-local /
   // 128 die-local / 128 plain): 1 Mi elements 3.40 / 3.42 / 3.68 / 3.74; 2 Mi 5.5 / 5.5 / 5.5 / 6.4;
   // 4 Mi 9.87 / 9.44 / 9.21 / 10.6; 8 Mi 17.5 / 17.1 / 16.8 / 18.5; 16 Mi 32.7 / 32.3 / 31.7 / 32.4;
@@ -208,7 +242,7 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
   // Both limits are in 256-vector tiles (4 KiB) of the largest segment.
   constexpr uint64_t kWg128MinTiles = 2049, kDieLocalMaxTiles = 32768;
   const uint64_t tiles = (*max_n / per_vec + 255) / 256;
-  shape->aligned = true;
+  shape->aligned = misfit == 0;
   shape->threads = tiles >= kWg128MinTiles ? 128 : 256;
   shape->die_local = tiles >= 64 && tiles <= kDieLocalMaxTiles;
   // Stores go through the memory-side cache while a launch writes at most half of its 256 MB
@@ -245,15 +279,11 @@ hipError_t LaunchSegments(const SegmentBatch& given, int dtype, hipStream_t stre
     }
   }
 
-  uint64_t blocks = (max_n / per_vec + kGeneralThreads - 1) / kGeneralThreads;
-  if (blocks == 0) blocks = 1;
-  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
   switch (dtype) {
-    case kF32: return LaunchGeneral<float, f32x4, uint32_t, u32x4>(batch, grid, add, stream);
-    case kI32: return LaunchGeneral<uint32_t, u32x4, uint32_t, u32x4>(batch, grid, add, stream);
-    case kF64: return LaunchGeneral<double, f64x2, uint64_t, u64x2>(batch, grid, add, stream);
-    case kI64: return LaunchGeneral<uint64_t, u64x2, uint64_t, u64x2>(batch, grid, add, stream);
+    case kF32: return LaunchPeeled<float, f32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream);
+    case kI32: return LaunchPeeled<uint32_t, u32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream);
+    case kF64: return LaunchPeeled<double, f64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream);
+    case kI64: return LaunchPeeled<uint64_t, u64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream);
     default: return hipErrorInvalidValue;
   }
 }

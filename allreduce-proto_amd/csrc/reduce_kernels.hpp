@@ -23,7 +23,8 @@
 // of its loads delays them; for launches of moderate size it also orders its tiles so that each
 // of the 8 dies works on runs of consecutive tiles.  SegmentKernel takes everything else (odd
 // offsets, ragged tails): a segment whose three pointers share their 16-byte phase is peeled at
-// head and tail so the body stays vectorised, any other segment runs element by element.
+// head and tail so the body stays vectorised, with the same workgroup size, tile order and store
+// policy; any other segment runs element by element.
 //
 // One workgroup per tile and nothing persistent, on purpose: on MI355X the hardware's own
 // in-order workgroup dispatch keeps the addresses in flight in one narrow moving window, and
@@ -46,9 +47,9 @@ namespace ibcomm_hip {
 // How a launch will be issued, for tests and the benchmark's report.
 struct LaunchShape {
   bool aligned;    // AlignedSegmentKernel (true) or SegmentKernel (false)
-  int threads;     // workgroup size: 256, or 128 for large aligned segments
-  bool die_local;  // aligned kernel only: tiles ordered so that each die gets runs of 8 consecutive tiles
-  bool write_through;  // aligned kernel only: stores written through the memory-side cache instead of past it
+  int threads;     // workgroup size: 256, or 128 for large segments
+  bool die_local;  // tiles ordered so that each die gets runs of 8 consecutive tiles
+  bool write_through;  // vector stores written through the memory-side cache instead of past it
   int segments;    // non-empty segments
 };
 

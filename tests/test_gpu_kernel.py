@@ -181,6 +181,77 @@ def test_aligned_segments_of_different_sizes_share_a_launch():
         assert torch.isnan(td[i][s:]).all(), "segment %d wrote past its end" % i
 
 
+@pytest.mark.parametrize("n", [1024 * 64 + 1, 1024 * 100 + 3, 1024 * 2048 - 1, 1024 * 2049 + 2, 1024 * 8192 - 1, 4194304 * 3 + 4194303,
+                               1024 * 32768 + 1, 1024 * 32769 + 3])
+@pytest.mark.parametrize("phase", [0, 1, 3])
+def test_peeled_kernel_geometries(n, phase):
+    # Off the 16-byte grid (operands `phase` elements into their buffers, lengths that are no whole number of
+    # vectors: config 5's ragged last ring step is 16,777,215 elements) the general kernel peels both ends and runs
+    # the aligned kernel's geometry in between: 128/256 threads, permuted tile order, either store policy.  Every
+    # element once, nothing outside, and the bits of the oracle's loop on a sampled stripe at each end.
+    g = torch.Generator(device="cuda").manual_seed(n + phase)
+    a = torch.randn(n + 8, device="cuda", generator=g)
+    b = torch.randn(n + 8, device="cuda", generator=g)
+    d = torch.full((n + 264,), float("nan"), device="cuda")
+    es = 4
+    torch.cuda.synchronize()
+    assert H.lib().ibcomm_hip_reduce(H.F32, d.data_ptr() + phase * es, a.data_ptr() + phase * es, b.data_ptr() + phase * es, n, None) == 0, H.last_error()
+    torch.cuda.synchronize()
+    want = a[phase:phase + n] + b[phase:phase + n]
+    assert torch.equal(d[phase:phase + n].view(torch.int32), want.view(torch.int32))
+    assert torch.isnan(d[:phase]).all() and torch.isnan(d[phase + n:]).all(), "wrote outside the segment"
+    for s in (slice(0, 4099), slice(n - 4099, n)):
+        ha, hb = a[phase:phase + n][s].cpu().numpy(), b[phase:phase + n][s].cpu().numpy()
+        assert np.array_equal(O.bits(d[phase:phase + n][s].cpu().numpy()), O.bits(oracle_add(ha, hb)))
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.float64, torch.int64])
+def test_peeled_kernel_other_types_adds_and_copies(dtype):
+    code = {torch.int32: H.I32, torch.float64: H.F64, torch.int64: H.I64}[dtype]
+    es = torch.empty(0, dtype=dtype).element_size()
+    for n in (1024 * 300 + 1, 1024 * 3000 + 1):
+        for phase in ((0, 1) if es == 8 else (0, 1, 2, 3)):
+            g = torch.Generator(device="cuda").manual_seed(n + phase)
+            a = torch.randint(-2**31, 2**31 - 1, (n + 4,), device="cuda", generator=g).to(dtype) if dtype != torch.float64 \
+                else torch.randn(n + 4, device="cuda", generator=g, dtype=dtype)
+            b = a.flip(0).clone()
+            d = torch.zeros(n + 8, dtype=dtype, device="cuda")
+            c = torch.zeros(n + 8, dtype=dtype, device="cuda")
+            o = phase * es
+            vp = C.c_void_p
+            torch.cuda.synchronize()
+            assert H.lib().ibcomm_hip_reduce(code, d.data_ptr() + o, a.data_ptr() + o, b.data_ptr() + o, n, None) == 0, H.last_error()
+            assert H.lib().ibcomm_hip_copy_segments(code, 1, (vp * 1)(c.data_ptr() + o), (vp * 1)(a.data_ptr() + o), (C.c_size_t * 1)(n), None) == 0, H.last_error()
+            torch.cuda.synchronize()
+            assert torch.equal(d[phase:phase + n], a[phase:phase + n] + b[phase:phase + n])
+            assert torch.equal(c[phase:phase + n], a[phase:phase + n])
+            for t in (d, c):
+                assert (t[:phase] == 0).all() and (t[phase + n:] == 0).all(), "wrote outside the segment"
+
+
+def test_peeled_segments_of_different_sizes_and_phases_share_a_launch():
+    # segments of one launch may each sit at their own 16-byte phase; those whose three operands do not share
+    # one go element by element in the same launch
+    sizes = [1024 * 3 + 1, 1024 * 2100 + 3, 1024 * 70, 0, 5, 1024 * 700 + 2, 1024 * 64 + 1]
+    phases = [(1, 1, 1), (2, 2, 2), (0, 0, 0), (0, 0, 0), (3, 3, 3), (1, 2, 3), (0, 3, 0)]
+    k = len(sizes)
+    g = torch.Generator(device="cuda").manual_seed(13)
+    ta = [torch.randn(s + 8, device="cuda", generator=g) for s in sizes]
+    tb = [torch.randn(s + 8, device="cuda", generator=g) for s in sizes]
+    td = [torch.full((s + 72,), float("nan"), device="cuda") for s in sizes]
+    vp = C.c_void_p
+    torch.cuda.synchronize()
+    rc = H.lib().ibcomm_hip_reduce_segments(H.F32, k, (vp * k)(*[t.data_ptr() + 4 * p[0] for t, p in zip(td, phases)]),
+                                            (vp * k)(*[t.data_ptr() + 4 * p[1] for t, p in zip(ta, phases)]),
+                                            (vp * k)(*[t.data_ptr() + 4 * p[2] for t, p in zip(tb, phases)]), (C.c_size_t * k)(*sizes), None)
+    assert rc == 0, H.last_error()
+    torch.cuda.synchronize()
+    for i, (s, p) in enumerate(zip(sizes, phases)):
+        want = ta[i][p[1]:p[1] + s] + tb[i][p[2]:p[2] + s]
+        assert torch.equal(td[i][p[0]:p[0] + s].view(torch.int32), want.view(torch.int32)), "segment %d" % i
+        assert torch.isnan(td[i][:p[0]]).all() and torch.isnan(td[i][p[0] + s:]).all(), "segment %d wrote outside" % i
+
+
 def test_large_linear_property():
     # 256 MiB operands: compare with torch's own fp32 add on the device (IEEE add, same rounding)
     n = 67108864

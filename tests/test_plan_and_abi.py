@@ -130,7 +130,8 @@ def test_launch_geometry_follows_the_segment_size():
     # The reference fixes 512 threads and min(ceil(n / 512), 65535) blocks for every size
     # (allreduce_cuda_impl.h:24, 116-117); here the aligned kernel runs one 16-byte vector per lane,
     # 256-thread workgroups up to 2 Mi fp32 per segment and 128 beyond, die-local tile order from 64 tiles
-    # up to 32 Mi fp32, and anything off the 16-byte grid goes to the general kernel.
+    # up to 32 Mi fp32, and anything off the 16-byte grid goes to the general kernel, which keeps that geometry
+    # around its peeled ends.
     import ctypes as C
     L = H.lib()
 
@@ -158,8 +159,10 @@ def test_launch_geometry_follows_the_segment_size():
     assert describe([33554432 + 1024]) == (1, 128, 0)  # beyond 32 Mi fp32 the plain order is the faster one
     assert describe([67108864]) == (1, 128, 0)
     assert describe([8388608], H.F64) == (1, 128, 1) and describe([1048576], H.F64) == (1, 256, 1)  # limits are in bytes
-    assert describe([4194303]) == (0, 256, 0)          # config 5's ragged last chunk: not a whole number of vectors
-    assert describe([8388608], base=(0x10000004, 0x20000004, 0x30000004)) == (0, 256, 0)  # off the 16-byte grid
+    assert describe([4194303]) == (0, 128, 1)          # config 5's ragged last chunk: not a whole number of vectors
+    assert describe([4194304, 4194304, 4194304, 4194303]) == (0, 128, 1)  # its whole last ring step
+    assert describe([8388608], base=(0x10000004, 0x20000004, 0x30000004)) == (0, 128, 1)  # off the 16-byte grid
+    assert describe([2521]) == (0, 256, 0)             # the reference tester's 2521 elements
     assert describe([0, 8388608, 0]) == (1, 128, 1)    # empty segments do not count
     assert describe([]) == (0, 256, 0)
     assert L.ibcomm_hip_describe_launch(7, 0, None, None, None, None, None, None, None, None) == H.INVALID_ARGUMENT
