@@ -189,7 +189,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches, sta
         # counter traffic is known for the kernel geometry it was collected on, and only for that
         "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value, through.value)) if aligned.value else None,
         "kernel": "ibcomm_hip::%s<float4, %d threads, add>, %s tile order, non-temporal loads, %s stores" % (
-            ("AlignedOneSegmentKernel" if k == 1 else "AlignedSegmentKernel") if aligned.value else "SegmentKernel", threads.value,
+            ("Aligned" if aligned.value else "") + ("OneSegmentKernel" if k == 1 else "SegmentKernel"), threads.value,
             "die-local" if die_local.value else "plain", "written-through (sc1)" if through.value else "non-temporal"),
         "launch_shape": shape,
         "algorithmic_bytes_per_launch": int(algorithmic),
