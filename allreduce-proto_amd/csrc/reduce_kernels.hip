@@ -234,10 +234,12 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
   }
   shape->segments = batch->count;
   if (*max_n == 0) return hipSuccess;
-  // Measured on MI355X with fp32 (us per launch of one segment, 256 threads plain / 256 die-local /
-  // 128 die-local / 128 plain): 1 Mi elements 3.40 / 3.42 / 3.68 / 3.74; 2 Mi 5.5 / 5.5 / 5.5 / 6.4;
-  // 4 Mi 9.87 / 9.44 / 9.21 / 10.6; 8 Mi 17.5 / 17.1 / 16.8 / 18.5; 16 Mi 32.7 / 32.3 / 31.7 / 32.4;
-  // 32 Mi 63.3 / 63.3 / 61.0 / 63.1; 64 Mi 125 / 129 / 122.2 / 122.1; 128 Mi 250 / 265 / 248 / 244.
+  // Measured on MI355X with fp32, one segment, non-temporal stores (us per launch: 256 threads plain /
+  // 256 die-local / 128 die-local / 128 plain): 1 Mi elements 3.40 / 3.42 / 3.68 / 3.74; 2 Mi 5.5 / 5.5 /
+  // 5.5 / 6.4; 4 Mi 9.87 / 9.44 / 9.21 / 10.6; 8 Mi 17.5 / 17.1 / 16.8 / 18.5; 16 Mi 32.7 / 32.3 / 31.7 /
+  // 32.4; 32 Mi 63.3 / 63.3 / 61.0 / 63.1; 64 Mi 125 / 129 / 122.2 / 122.1; 128 Mi 250 / 265 / 248 / 244.
+  // With written-through stores the two workgroup sizes are closer (256 / 128 threads, die-local: 1 Mi
+  // 3.36 / 3.38; 2 Mi 4.94 / 4.87; 4 Mi 8.52 / 8.49; 8 Mi 15.37 / 15.18; 12 Mi 22.10 / 21.86), same order.
   // Hence: 256 threads up to 2 Mi elements, 128 beyond; die-local tile order up to 32 Mi elements.
   // Both limits are in 256-vector tiles (4 KiB) of the largest segment.
   constexpr uint64_t kWg128MinTiles = 2049, kDieLocalMaxTiles = 32768;
