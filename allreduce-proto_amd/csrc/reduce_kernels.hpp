@@ -22,9 +22,9 @@
 // with one vector per lane a workgroup lives for one memory round trip and every instruction ahead
 // of its loads delays them; for launches of moderate size it also orders its tiles so that each
 // of the 8 dies works on runs of consecutive tiles.  SegmentKernel takes everything else (odd
-// offsets, ragged tails): a segment whose three pointers share their 16-byte phase is peeled at
-// head and tail so the body stays vectorised, with the same workgroup size, tile order and store
-// policy; any other segment runs element by element.
+// offsets, ragged tails): a segment is peeled at head and tail so that the body runs in 16-byte
+// vectors on dst's grid, with the same workgroup size, tile order and store policy; operands at
+// another 16-byte phase are loaded as vectors from element-aligned addresses.
 //
 // One workgroup per tile and nothing persistent, on purpose: on MI355X the hardware's own
 // in-order workgroup dispatch keeps the addresses in flight in one narrow moving window, and

@@ -252,6 +252,47 @@ def test_peeled_segments_of_different_sizes_and_phases_share_a_launch():
         assert torch.isnan(td[i][:p[0]]).all() and torch.isnan(td[i][p[0] + s:]).all(), "segment %d wrote outside" % i
 
 
+@pytest.mark.parametrize("n", [1024 * 100 + 3, 1024 * 2049 + 2, 1024 * 8192 - 1])
+@pytest.mark.parametrize("phases", [(1, 2, 3), (0, 3, 0), (2, 0, 1), (0, 0, 1)])
+def test_operands_at_different_phases_at_every_geometry(n, phases):
+    # dst, a and b each at their own 4-byte phase: the vector body follows dst's 16-byte grid and the
+    # operands are loaded as 16-byte vectors from element-aligned addresses
+    pd, pa, pb = phases
+    g = torch.Generator(device="cuda").manual_seed(n + pd * 16 + pa * 4 + pb)
+    a = torch.randn(n + 8, device="cuda", generator=g)
+    b = torch.randn(n + 8, device="cuda", generator=g)
+    d = torch.full((n + 264,), float("nan"), device="cuda")
+    torch.cuda.synchronize()
+    assert H.lib().ibcomm_hip_reduce(H.F32, d.data_ptr() + 4 * pd, a.data_ptr() + 4 * pa, b.data_ptr() + 4 * pb, n, None) == 0, H.last_error()
+    torch.cuda.synchronize()
+    want = a[pa:pa + n] + b[pb:pb + n]
+    assert torch.equal(d[pd:pd + n].view(torch.int32), want.view(torch.int32))
+    assert torch.isnan(d[:pd]).all() and torch.isnan(d[pd + n:]).all(), "wrote outside the segment"
+    # the copy of the same shape
+    c = torch.full((n + 264,), float("nan"), device="cuda")
+    vp = C.c_void_p
+    assert H.lib().ibcomm_hip_copy_segments(H.F32, 1, (vp * 1)(c.data_ptr() + 4 * pd), (vp * 1)(a.data_ptr() + 4 * pa), (C.c_size_t * 1)(n), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(c[pd:pd + n].view(torch.int32), a[pa:pa + n].view(torch.int32))
+    assert torch.isnan(c[:pd]).all() and torch.isnan(c[pd + n:]).all(), "the copy wrote outside the segment"
+
+
+def test_eight_byte_operands_at_different_phases():
+    for dtype, code in ((torch.float64, H.F64), (torch.int64, H.I64)):
+        for n in (1024 * 50 + 1, 1024 * 3000 + 1):
+            for pd, pa, pb in ((0, 1, 0), (1, 0, 1), (1, 0, 0)):
+                g = torch.Generator(device="cuda").manual_seed(n + pd + 2 * pa + 4 * pb)
+                a = torch.randn(n + 4, device="cuda", generator=g, dtype=torch.float64)
+                a = a if dtype == torch.float64 else (a * 1e15).to(torch.int64)
+                b = a.flip(0).clone()
+                d = torch.zeros(n + 8, dtype=dtype, device="cuda")
+                torch.cuda.synchronize()
+                assert H.lib().ibcomm_hip_reduce(code, d.data_ptr() + 8 * pd, a.data_ptr() + 8 * pa, b.data_ptr() + 8 * pb, n, None) == 0, H.last_error()
+                torch.cuda.synchronize()
+                assert torch.equal(d[pd:pd + n], a[pa:pa + n] + b[pb:pb + n])
+                assert (d[:pd] == 0).all() and (d[pd + n:] == 0).all(), "wrote outside the segment"
+
+
 def test_large_linear_property():
     # 256 MiB operands: compare with torch's own fp32 add on the device (IEEE add, same rounding)
     n = 67108864
