@@ -53,9 +53,11 @@ __device__ __forceinline__ uint64_t TileOf(uint32_t block, uint32_t die_local_ti
 
 // Any alignment, any length.  T is the element type, V the 16-byte vector of T.  Integer types
 // are instantiated unsigned so that += wraps.  ADD selects dst = a + b; otherwise the launch is a
-// copy, dst = a.  A segment is peeled: up to 16 bytes element by element until dst reaches a 16-byte
-// boundary, 16-byte vectors from there, the rest element by element, with the tile order and the
-// store policy of the aligned kernel.  Operands that do not share dst's 16-byte phase are loaded as
+// copy, dst = a.  A segment is peeled: element by element until dst reaches a 128-byte boundary
+// (so that a wave's kilobyte of stores covers whole cache lines: starting at the first 16-byte
+// boundary instead leaves every wave a partial line at each end and costs 4 % at 8 Mi fp32),
+// 16-byte vectors from there, the rest element by element, with the tile order and the store
+// policy of the aligned kernel.  Operands that do not share dst's 16-byte phase are loaded as
 // 16-byte vectors all the same, from addresses that are only element-aligned (gfx950 takes those
 // in its global memory instructions).  Only pointers that are not even element-aligned send a
 // segment through the element loop as a whole.
@@ -63,6 +65,7 @@ template <typename T, typename V, int THREADS, bool ADD>
 __device__ __forceinline__ void PeeledTile(T* dst, const T* a, const T* b, uint64_t n, uint32_t die_local_tiles, uint32_t write_through) {
   typedef V ElementAlignedV __attribute__((aligned(sizeof(T))));
   constexpr uint64_t kPerVec = 16 / sizeof(T);
+  constexpr uintptr_t kHeadAlign = 128;
   const uintptr_t pd = reinterpret_cast<uintptr_t>(dst) & 15;
   const uintptr_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(a) | (ADD ? reinterpret_cast<uintptr_t>(b) : 0);
   const bool same_phase = ((reinterpret_cast<uintptr_t>(a) & 15) == pd) && (!ADD || (reinterpret_cast<uintptr_t>(b) & 15) == pd);
@@ -70,7 +73,7 @@ __device__ __forceinline__ void PeeledTile(T* dst, const T* a, const T* b, uint6
   // [0, head) scalar, [head, head + nvec * kPerVec) as 16-byte vectors, rest scalar.
   uint64_t head = n, nvec = 0;
   if (all % sizeof(T) == 0) {
-    head = ((16 - pd) & 15) / sizeof(T);
+    head = ((kHeadAlign - (reinterpret_cast<uintptr_t>(dst) & (kHeadAlign - 1))) & (kHeadAlign - 1)) / sizeof(T);
     if (head > n) head = n;
     nvec = (n - head) / kPerVec;
   }
@@ -89,7 +92,7 @@ __device__ __forceinline__ void PeeledTile(T* dst, const T* a, const T* b, uint6
     else __builtin_nontemporal_store(v, reinterpret_cast<V*>(dst + head) + i);
   }
 
-  // Scalar remainder: fewer than two vectors' worth, or the whole segment.
+  // Scalar remainder: less than 128 + 16 bytes, or the whole segment.
   const uint64_t tail_begin = head + nvec * kPerVec;
   const uint64_t scalar_count = head + (n - tail_begin);
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * THREADS;
