@@ -17,7 +17,7 @@
 // through to the memory-side cache.
 //
 // Two kernels share that contract.  AlignedSegmentKernel takes the launches in which every pointer
-// is on a 16-byte boundary and every length a whole number of vectors (in practice all of the
+// is on a 16-byte boundary (dst on a 128-byte one) and every length a whole number of vectors (in practice all of the
 // engine's, since chunk sizes and buffers are aligned): load, add, store, nothing else, because
 // with one vector per lane a workgroup lives for one memory round trip and every instruction ahead
 // of its loads delays them; for launches of moderate size it also orders its tiles so that each

@@ -163,6 +163,8 @@ def test_launch_geometry_follows_the_segment_size():
     assert describe([4194304, 4194304, 4194304, 4194303]) == (0, 128, 1)  # its whole last ring step
     assert describe([8388608], base=(0x10000004, 0x20000004, 0x30000004)) == (0, 128, 1)  # off the 16-byte grid
     assert describe([2521]) == (0, 256, 0)             # the reference tester's 2521 elements
+    assert describe([8388608], base=(0x10000010, 0x20000000, 0x30000000)) == (0, 128, 1)  # dst off the 128-byte grid
+    assert describe([8388608], base=(0x10000080, 0x20000010, 0x30000020)) == (1, 128, 1)  # operands need 16 bytes only
     assert describe([0, 8388608, 0]) == (1, 128, 1)    # empty segments do not count
     assert describe([]) == (0, 256, 0)
     assert L.ibcomm_hip_describe_launch(7, 0, None, None, None, None, None, None, None, None) == H.INVALID_ARGUMENT
