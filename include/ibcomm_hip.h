@@ -140,7 +140,10 @@ int ibcomm_hip_world_allreduce_noalloc(int world_size, int algo, int dtype, cons
  * paced as in the recorded run, and whose receives cost nothing.  Same result in recvbuf as the
  * world run gives that rank (for the same sendbuf contents).  This is how one GPU's part of
  * AllreduceRingCuda / AllreduceRabenseifnerCuda (ibcomm/allreduce_cuda_impl.h:35-301, 326-717) is
- * timed without the other ranks' work on the same device; the reference has no counterpart. */
+ * timed without the other ranks' work on the same device; the reference has no counterpart.
+ * Like ibcomm_hip_world_allreduce these two drive a fabric from one host thread: calls on one fabric
+ * must not overlap in time (the recording, the graph cache and the completion word belong to the
+ * fabric). */
 int ibcomm_hip_world_record(ibcomm_hip_comm* const* comms, int world_size, int rank, int algo, int dtype,
                             const void* const* sendbufs, void* const* recvbufs, size_t len_elements);
 int ibcomm_hip_replay_allreduce(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf,
@@ -169,7 +172,7 @@ int ibcomm_hip_max_segments(void);
 int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const void* const* src,
                              const size_t* len_elements, void* stream);
 /* How ibcomm_hip_reduce_segments would issue these segments, without launching: *aligned = 1 for the
- * kernel that takes 16-byte aligned pointers and whole vectors (0: the general kernel), *threads the
+ * kernel that takes 16-byte aligned pointers (dst: 128-byte aligned) and whole vectors (0: the general kernel), *threads the
  * workgroup size, *die_local = 1 if tiles are ordered in runs per accelerator die, *write_through = 1
  * if the stores go through the memory-side cache (0: non-temporal).  Stands for the launch geometry
  * the reference fixes at ibcomm/allreduce_cuda_impl.h:24, 116-117. */
