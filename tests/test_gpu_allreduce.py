@@ -96,6 +96,53 @@ def test_odd_chunk_offsets_keep_vector_path_correct():
         G.check_against_oracle(w, H.RING, rand_bufs(5, 1003))
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_worlds_lengths_chunks_and_buffer_phases(seed):
+    # Seeded draws over everything a caller can vary at once: algorithm, world size, odd lengths, chunk size,
+    # landing mode, chunks per launch, element type, and the 4-byte phase of every rank's sendbuf and recvbuf
+    # (each its own, so the three operands of a reduction can sit at three different phases).
+    rng = np.random.default_rng(1000 + seed)
+    algo = H.RING if rng.integers(2) else H.RABENSEIFNER
+    world = int(rng.choice([2, 3, 4, 5, 7, 8]) if algo == H.RING else rng.choice([2, 4, 8, 16]))
+    n = int(rng.integers(world, 300000))
+    dtype = [np.float32, np.int32, np.float64][int(rng.integers(3))]
+    es = np.dtype(dtype).itemsize
+    chunk = None
+    if rng.integers(2):
+        per = int(rng.integers(1, max(2, n // (2 * world) + 1)))  # elements per chunk, at least 2 * world chunks
+        if (n + per - 1) // per >= 2 * world:
+            chunk = per * es
+    if dtype == np.int32:
+        host = [rng.integers(-2**31, 2**31 - 1, n, dtype=np.int64).astype(np.int32) for _ in range(world)]
+    else:
+        host = [(rng.standard_normal(n) * 10.0 ** float(rng.integers(-3, 3))).astype(dtype) for _ in range(world)]
+    tdt = G.TORCH_DT[G.NP_TO_H[np.dtype(dtype)]]
+    send_off = [int(rng.integers(4)) for _ in range(world)]
+    recv_off = [int(rng.integers(4)) for _ in range(world)]
+    send_t = [torch.zeros(n + 8, dtype=tdt, device="cuda") for _ in range(world)]
+    recv_t = [torch.full((n + 8,), 85, dtype=tdt, device="cuda") for _ in range(world)]
+    for r in range(world):
+        send_t[r][send_off[r]:send_off[r] + n] = torch.from_numpy(host[r]).cuda()
+    with H.World(world) as w:
+        w.set_landing(int(rng.choice([H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])))
+        w.set_max_fuse(int(rng.choice([1, 3, 16, 64])))
+        torch.cuda.synchronize()
+        for call in range(3):  # eager, recorded, replayed
+            with G.env(IBCOMM_CHUNKSIZE=chunk):
+                rc = w.allreduce_ptrs(algo, G.NP_TO_H[np.dtype(dtype)], [t.data_ptr() + o * es for t, o in zip(send_t, send_off)],
+                                      [t.data_ptr() + o * es for t, o in zip(recv_t, recv_off)], n)
+            assert rc == 0, "seed %d call %d: %s" % (seed, call, H.last_error())
+            torch.cuda.synchronize()
+            orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
+            assert orc == 0
+            for r in range(world):
+                got = recv_t[r].cpu().numpy()
+                o = recv_off[r]
+                assert np.array_equal(O.bits(got[o:o + n]), O.bits(want[r])), "seed %d call %d rank %d" % (seed, call, r)
+                assert (got[:o] == 85).all() and (got[o + n:] == 85).all(), "seed %d rank %d wrote outside recvbuf" % (seed, r)
+                recv_t[r][o:o + n] = 85
+
+
 @pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 4, None), (H.RING, 8, 4096), (H.RABENSEIFNER, 8, None)])
 def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
