@@ -10,6 +10,7 @@
 
 #include "backend_hip.hpp"
 #include "engine.hpp"
+#include "rendezvous.hpp"
 #include "world.hpp"
 
 using namespace ibcomm_hip;
@@ -52,11 +53,13 @@ __global__ void PublishCompletion(uint64_t* host_flag) {
 }
 
 struct ibcomm_hip_fabric {
-  explicit ibcomm_hip_fabric(int n) : fabric(n) {
+  explicit ibcomm_hip_fabric(int n) : fabric(n), meet(n) {
     const char* v = getenv("IBCOMM_HIP_GRAPH");
     graph_mode = v ? atoi(v) : 1;
     v = getenv("IBCOMM_HIP_GRAPH_MAX_OPS");
     graph_max_ops = v ? strtoull(v, nullptr, 10) : 4096;
+    v = getenv("IBCOMM_HIP_RENDEZVOUS");
+    meet_mode = v ? atoi(v) : 1;
   }
   ~ibcomm_hip_fabric() {
     DropGraphs();
@@ -65,7 +68,10 @@ struct ibcomm_hip_fabric {
     if (timer[0]) (void)hipEventDestroy(timer[0]);
     if (timer[1]) (void)hipEventDestroy(timer[1]);
   }
+  // A replay returns when its last node has published the completion word, which can be a moment
+  // before the runtime has retired the launch: let it, before an executable graph goes away.
   void DropGraphs() {
+    if (origin && !graphs.empty()) (void)hipStreamSynchronize(origin);
     for (CachedGraph& g : graphs) {
       if (g.exec) (void)hipGraphExecDestroy(g.exec);
       if (g.graph) (void)hipGraphDestroy(g.graph);
@@ -73,6 +79,8 @@ struct ibcomm_hip_fabric {
     graphs.clear();
   }
   Fabric<HipBackend> fabric;
+  Rendezvous meet;               // where the blocking per-rank calls of this world find each other
+  int meet_mode = 1;             // 0 = every rank thread runs its own engine (IBCOMM_HIP_RENDEZVOUS=0)
   std::mutex mu;                 // guards live_comms and the graph cache against concurrent create / destroy
   int live_comms = 0;
   int graph_mode = 1;            // 0 = always issue eagerly, 1 = capture a call shape on its second use
@@ -160,65 +168,6 @@ int ibcomm_hip_comm_register_myself(ibcomm_hip_comm* comm, int my_rank) {
     return Fail(kInvalidArgument, "rank %d outside world of %d", my_rank, comm->comm.world_size());
   comm->comm.RegisterMyself(my_rank);
   return kOk;
-}
-
-int ibcomm_hip_allreduce_ring(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
-  if (!comm) return Fail(kInvalidArgument, "comm is null");
-  return comm->comm.AllreduceBlocking(kRing, dtype, sendbuf, recvbuf, len);
-}
-
-int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
-  if (!comm) return Fail(kInvalidArgument, "comm is null");
-  return comm->comm.AllreduceBlocking(kRabenseifner, dtype, sendbuf, recvbuf, len);
-}
-
-}  // extern "C"
-
-namespace {
-// Host buffers in, host buffers out: copy up, run the device collective, copy down.
-int AllreduceHost(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
-  if (!comm) return Fail(kInvalidArgument, "comm is null");
-  const size_t es = DTypeSize(dtype);
-  if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
-  if (!sendbuf || !recvbuf) return Fail(kInvalidArgument, "sendbuf and recvbuf must not be null");
-  const size_t bytes = len * es;
-  if (bytes > comm->stage_bytes) {
-    if (comm->stage_send) IBCOMM_HIP_CHECK(hipFree(comm->stage_send));
-    if (comm->stage_recv) IBCOMM_HIP_CHECK(hipFree(comm->stage_recv));
-    comm->stage_send = comm->stage_recv = nullptr;
-    comm->stage_bytes = 0;
-    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_send, bytes));
-    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_recv, bytes));
-    comm->stage_bytes = bytes;
-  }
-  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(comm->stage_send, sendbuf, bytes, hipMemcpyHostToDevice));
-  IBCOMM_RETURN_IF_ERROR(comm->comm.AllreduceBlocking(algo, dtype, comm->stage_send ? comm->stage_send : sendbuf,
-                                                      comm->stage_recv ? comm->stage_recv : recvbuf, len));
-  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(recvbuf, comm->stage_recv, bytes, hipMemcpyDeviceToHost));
-  return kOk;
-}
-}  // namespace
-
-extern "C" {
-
-int ibcomm_hip_allreduce_ring_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
-  return AllreduceHost(comm, kRing, dtype, sendbuf, recvbuf, len);
-}
-int ibcomm_hip_allreduce_rabenseifner_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
-  return AllreduceHost(comm, kRabenseifner, dtype, sendbuf, recvbuf, len);
-}
-
-int ibcomm_hip_allreduce_ring_f32(ibcomm_hip_comm* c, const float* s, float* r, size_t n) {
-  return ibcomm_hip_allreduce_ring(c, kF32, s, r, n);
-}
-int ibcomm_hip_allreduce_ring_i32(ibcomm_hip_comm* c, const int32_t* s, int32_t* r, size_t n) {
-  return ibcomm_hip_allreduce_ring(c, kI32, s, r, n);
-}
-int ibcomm_hip_allreduce_rabenseifner_f32(ibcomm_hip_comm* c, const float* s, float* r, size_t n) {
-  return ibcomm_hip_allreduce_rabenseifner(c, kF32, s, r, n);
-}
-int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* c, const int32_t* s, int32_t* r, size_t n) {
-  return ibcomm_hip_allreduce_rabenseifner(c, kI32, s, r, n);
 }
 
 }  // extern "C"
@@ -352,6 +301,7 @@ int IssueCached(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs
       return rc;
     }
     if (f->graphs.size() >= kMaxCachedGraphs) {
+      (void)hipStreamSynchronize(f->origin);  // a replay returns on its completion word, possibly before the runtime has retired it
       (void)hipGraphExecDestroy(f->graphs.front().exec);
       (void)hipGraphDestroy(f->graphs.front().graph);
       f->graphs.erase(f->graphs.begin());
@@ -400,16 +350,11 @@ int CollectWorld(ibcomm_hip_comm* const* comms, int world_size, std::vector<Comm
   return kOk;
 }
 
-}  // namespace
-
-extern "C" {
-
-int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
-                               const void* const* sendbufs, void* const* recvbufs, size_t len) {
-  if (!comms || !sendbufs || !recvbufs || world_size < 1) return Fail(kInvalidArgument, "null argument");
-  std::vector<Communicator<HipBackend>*> cs;
-  IBCOMM_RETURN_IF_ERROR(CollectWorld(comms, world_size, &cs));
-  ibcomm_hip_fabric* f = comms[0]->owner;
+// One allreduce of the whole world from the calling thread: eager on the first use of a call shape,
+// recorded on the second, replayed from then on.
+int WorldAllreduce(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>& cs, int algo, int dtype,
+                   const void* const* sendbufs, void* const* recvbufs, size_t len) {
+  const int world_size = static_cast<int>(cs.size());
   // Recording hipMemcpyAsync device-to-device copies into a graph crashed the host process inside
   // the runtime on ROCm 7.2 (gfx950), so the per-message-memcpy landing mode is never recorded.
   const bool may_record = f->graph_mode != 0 && world_size > 1 && cs[0]->landing() != kLandMemcpy;
@@ -417,6 +362,101 @@ int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, in
   return IssueCached(f, cs, key, may_record, [&](bool synchronize) {
     return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, synchronize);
   });
+}
+
+double TimeLimitSeconds() {
+  const char* t = getenv("IBCOMM_HIP_TIMEOUT_S");
+  return t ? atof(t) : 120.0;
+}
+
+// The blocking per-rank call, the shape of AllreduceRingCuda / AllreduceRabenseifnerCuda.  The
+// ranks of a world meet (rendezvous.hpp): the last to arrive runs the collective for all of them
+// through the single-thread driver above, so the reference's own entry point gets the recorded
+// graph.  With IBCOMM_HIP_RENDEZVOUS=0 every rank thread runs its own engine instead and the
+// ranks exchange messages as separate processes would.
+int BlockingAllreduce(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  ibcomm_hip_fabric* f = comm->owner;
+  const int world_size = comm->comm.world_size();
+  if (world_size == 1 || f->meet_mode == 0) return comm->comm.AllreduceBlocking(algo, dtype, sendbuf, recvbuf, len);
+  RankCall call;
+  call.comm = &comm->comm;
+  call.algo = algo;
+  call.dtype = dtype;
+  call.sendbuf = sendbuf;
+  call.recvbuf = recvbuf;
+  call.len = len;
+  return f->meet.Arrive(comm->comm.rank(), call, TimeLimitSeconds(), &f->fabric, [f, world_size](const RankCall* calls) {
+    std::vector<Communicator<HipBackend>*> cs(world_size);
+    std::vector<const void*> sends(world_size);
+    std::vector<void*> recvs(world_size);
+    for (int r = 0; r < world_size; r++) {
+      cs[r] = static_cast<Communicator<HipBackend>*>(calls[r].comm);
+      sends[r] = calls[r].sendbuf;
+      recvs[r] = calls[r].recvbuf;
+    }
+    return WorldAllreduce(f, cs, calls[0].algo, calls[0].dtype, sends.data(), recvs.data(), calls[0].len);
+  });
+}
+
+// Host buffers in, host buffers out: copy up, run the device collective, copy down.
+int AllreduceHost(ibcomm_hip_comm* comm, int algo, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  if (!comm) return Fail(kInvalidArgument, "comm is null");
+  const size_t es = DTypeSize(dtype);
+  if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
+  if (!sendbuf || !recvbuf) return Fail(kInvalidArgument, "sendbuf and recvbuf must not be null");
+  const size_t bytes = len * es;
+  if (bytes > comm->stage_bytes) {
+    if (comm->stage_send) IBCOMM_HIP_CHECK(hipFree(comm->stage_send));
+    if (comm->stage_recv) IBCOMM_HIP_CHECK(hipFree(comm->stage_recv));
+    comm->stage_send = comm->stage_recv = nullptr;
+    comm->stage_bytes = 0;
+    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_send, bytes));
+    IBCOMM_HIP_CHECK(hipMalloc(&comm->stage_recv, bytes));
+    comm->stage_bytes = bytes;
+  }
+  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(comm->stage_send, sendbuf, bytes, hipMemcpyHostToDevice));
+  IBCOMM_RETURN_IF_ERROR(BlockingAllreduce(comm, algo, dtype, comm->stage_send ? comm->stage_send : sendbuf,
+                                           comm->stage_recv ? comm->stage_recv : recvbuf, len));
+  if (bytes) IBCOMM_HIP_CHECK(hipMemcpy(recvbuf, comm->stage_recv, bytes, hipMemcpyDeviceToHost));
+  return kOk;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ibcomm_hip_allreduce_ring(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return BlockingAllreduce(comm, kRing, dtype, sendbuf, recvbuf, len);
+}
+int ibcomm_hip_allreduce_rabenseifner(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return BlockingAllreduce(comm, kRabenseifner, dtype, sendbuf, recvbuf, len);
+}
+int ibcomm_hip_allreduce_ring_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return AllreduceHost(comm, kRing, dtype, sendbuf, recvbuf, len);
+}
+int ibcomm_hip_allreduce_rabenseifner_host(ibcomm_hip_comm* comm, int dtype, const void* sendbuf, void* recvbuf, size_t len) {
+  return AllreduceHost(comm, kRabenseifner, dtype, sendbuf, recvbuf, len);
+}
+int ibcomm_hip_allreduce_ring_f32(ibcomm_hip_comm* c, const float* s, float* r, size_t n) {
+  return BlockingAllreduce(c, kRing, kF32, s, r, n);
+}
+int ibcomm_hip_allreduce_ring_i32(ibcomm_hip_comm* c, const int32_t* s, int32_t* r, size_t n) {
+  return BlockingAllreduce(c, kRing, kI32, s, r, n);
+}
+int ibcomm_hip_allreduce_rabenseifner_f32(ibcomm_hip_comm* c, const float* s, float* r, size_t n) {
+  return BlockingAllreduce(c, kRabenseifner, kF32, s, r, n);
+}
+int ibcomm_hip_allreduce_rabenseifner_i32(ibcomm_hip_comm* c, const int32_t* s, int32_t* r, size_t n) {
+  return BlockingAllreduce(c, kRabenseifner, kI32, s, r, n);
+}
+
+int ibcomm_hip_world_allreduce(ibcomm_hip_comm* const* comms, int world_size, int algo, int dtype,
+                               const void* const* sendbufs, void* const* recvbufs, size_t len) {
+  if (!comms || !sendbufs || !recvbufs || world_size < 1) return Fail(kInvalidArgument, "null argument");
+  std::vector<Communicator<HipBackend>*> cs;
+  IBCOMM_RETURN_IF_ERROR(CollectWorld(comms, world_size, &cs));
+  return WorldAllreduce(comms[0]->owner, cs, algo, dtype, sendbufs, recvbufs, len);
 }
 
 int ibcomm_hip_world_record(ibcomm_hip_comm* const* comms, int world_size, int rank, int algo, int dtype,

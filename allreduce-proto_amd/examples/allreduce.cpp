@@ -1,6 +1,6 @@
 // Loopback counterpart of PFNProto's example program (examples/allreduce.cpp).
 //
-//   allreduce_example [np [algorithm [elements]]]        defaults: 8 ring 67108864
+//   allreduce_example [np [algorithm [elements [timed_runs]]]]        defaults: 8 ring 67108864 1
 //
 // The reference runs one MPI process per rank; here the <np> ranks are threads of one process that
 // share the GPU, each with its own IBVerbsCommunicator and its own device buffers.  What each rank
@@ -9,6 +9,8 @@
 // last run (:28-29, :107-118), compare every element with the exact sum within 1e-6 (:130-140,
 // where the reference takes the answer from MPI_Allreduce), print "rank: r OK" or "rank: r FAIL"
 // and, once, "elapsed time : ... [s]" of rank 0.  The exit status is the number of failed ranks.
+// With timed_runs > 1 the collective runs that many more times after the warm-ups; the reference's
+// line still reports the first timed run and a second line lists rank 0's time for every one of them.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -40,7 +42,7 @@ void HipOrDie(hipError_t e, int line) {
 struct Rank {
   std::unique_ptr<IBVerbsCommunicator> comm;
   std::vector<float> send, recv;
-  double elapsed = 0;
+  std::vector<double> elapsed;  // per timed run
   bool ok = false;
 };
 
@@ -50,8 +52,9 @@ int main(int argc, char* argv[]) {
   const int np = argc > 1 ? atoi(argv[1]) : 8;
   const bool ring = argc > 2 ? strcmp(argv[2], "rabenseifner") != 0 : true;
   const size_t n = argc > 3 ? strtoull(argv[3], nullptr, 10) : 67108864ull;
-  if (np < 1 || n == 0 || (argc > 2 && strcmp(argv[2], "ring") && strcmp(argv[2], "rabenseifner"))) {
-    fprintf(stderr, "usage: %s [np [ring|rabenseifner [elements]]]\n", argv[0]);
+  const int timed_runs = argc > 4 ? atoi(argv[4]) : 1;
+  if (np < 1 || n == 0 || timed_runs < 1 || (argc > 2 && strcmp(argv[2], "ring") && strcmp(argv[2], "rabenseifner"))) {
+    fprintf(stderr, "usage: %s [np [ring|rabenseifner [elements [timed_runs]]]]\n", argv[0]);
     return 1;
   }
 
@@ -86,11 +89,11 @@ int main(int argc, char* argv[]) {
       HipOrDie(hipMalloc(reinterpret_cast<void**>(&dev_send), n * sizeof(float)), __LINE__);
       HipOrDie(hipMalloc(reinterpret_cast<void**>(&dev_recv), n * sizeof(float)), __LINE__);
       HipOrDie(hipMemcpy(dev_send, me.send.data(), n * sizeof(float), hipMemcpyHostToDevice), __LINE__);
-      for (int it = 0; it < kWarmup + 1; it++) {
+      for (int it = 0; it < kWarmup + timed_runs; it++) {
         const double start = Now();
         if (ring) me.comm->AllreduceRingCuda(dev_send, dev_recv, n);
         else me.comm->AllreduceRabenseifnerCuda(dev_send, dev_recv, n);
-        me.elapsed = Now() - start;
+        if (it >= kWarmup) me.elapsed.push_back(Now() - start);
       }
       HipOrDie(hipMemcpy(me.recv.data(), dev_recv, n * sizeof(float), hipMemcpyDeviceToHost), __LINE__);
       HipOrDie(hipFree(dev_send), __LINE__);
@@ -113,7 +116,12 @@ int main(int argc, char* argv[]) {
     printf("rank: %d%s\n", r, ranks[r].ok ? " OK" : " FAIL");
     failed += ranks[r].ok ? 0 : 1;
   }
-  printf("elapsed time : %e [s]\n", ranks[0].elapsed);
+  printf("elapsed time : %e [s]\n", ranks[0].elapsed[0]);
+  if (timed_runs > 1) {
+    printf("elapsed times of %d timed runs [s] :", timed_runs);
+    for (double t : ranks[0].elapsed) printf(" %e", t);
+    printf("\n");
+  }
   ranks.clear();
   return failed;
 }

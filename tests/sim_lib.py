@@ -48,7 +48,9 @@ DT = {np.dtype(np.float32): 0, np.dtype(np.int32): 1, np.dtype(np.float64): 2, n
 
 def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, threaded=False, repeats=1,
               pool_bytes=1 << 16, in_place=False, streams=None, copy=True):
-    """-> (rc, [recvbuf per rank], Report).  Environment knobs are set for the duration of the call."""
+    """-> (rc, [recvbuf per rank], Report).  Environment knobs are set for the duration of the call.
+    threaded: False = one thread steps all ranks, True (1) = one thread per rank, each with its own engine,
+    2 = one thread per rank, the blocking calls meet and the last to arrive steps all ranks."""
     world = len(sendbufs)
     if copy:  # copy=False: run on the caller's arrays, whatever their alignment
         sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]
@@ -74,7 +76,7 @@ def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, th
             os.environ["IBCOMM_NUM_CUDA_STREAM"] = str(streams)
         rep = Report()
         rc = lib().sim_world_allreduce(algo, DT[sendbufs[0].dtype], world, sp, rp, n, max_fuse, landing, seed,
-                                       1 if threaded else 0, repeats, C.byref(rep))
+                                       int(threaded), repeats, C.byref(rep))
     finally:
         for k, v in saved.items():
             if v is None:

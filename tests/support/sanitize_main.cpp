@@ -1,8 +1,9 @@
 // Stand-alone driver that runs the allreduce engine on the simulated device under the host
 // sanitizers (built by tests/test_engine_sanitizers.py with -fsanitize=address,undefined or
 // -fsanitize=thread; no GPU, no Python in the process).  Random worlds, lengths, chunk sizes, fusion
-// limits, landing modes and pool sizes, single-threaded lockstep and one thread per rank, plus the
-// record/replay, failure-handling and point-to-point cases of sim_world.cpp.
+// limits, landing modes and pool sizes, single-threaded lockstep, one thread per rank with an engine of
+// its own, and one thread per rank whose blocking calls meet (every other threaded world), plus the
+// record/replay, failure-handling, meeting and point-to-point cases of sim_world.cpp.
 //
 //   sanitize_main <iterations> <all_threaded 0|1> [<extras 0|1>]    exit status 0 if every run returned success
 // (extras, default 1: the failure-handling and point-to-point cases)
@@ -17,6 +18,7 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
 int sim_record_replay(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,
                       int rank, int max_fuse, int landing, unsigned seed, void* replay_out, int replays, void* rep);
 int sim_failures(void);
+int sim_rendezvous(void);
 int sim_p2p(void);
 }
 
@@ -50,7 +52,7 @@ int main(int argc, char** argv) {
       rp[i] = recv[i].data();
     }
     const int fuse = (rng() % 2) ? 64 : 1 + rng() % 64, landing = rng() % 4;
-    const int threaded = all_threaded || rng() % 5 == 0;
+    const int threaded = (all_threaded || rng() % 5 == 0) ? 1 + it % 2 : 0;
     int rc = sim_world_allreduce(algo, 0, world, sp.data(), rp.data(), n, fuse, landing, it, threaded, 1 + rng() % 2, report);
     runs++;
     if (rc != 0) {
@@ -70,9 +72,11 @@ int main(int argc, char** argv) {
   unsetenv("IBCOMM_CHUNKSIZE");
   unsetenv("IBCOMM_MEMORY_POOL_PRE_ALLOC");
   const int failures_held = extras ? sim_failures() : 4095, p2p_held = extras ? sim_p2p() : 2047;
-  if (failures_held != 4095 || p2p_held != 2047) {
+  const int meeting_held = sim_rendezvous();  // threads by nature: also in the run that skips the other extras
+  if (failures_held != 4095 || p2p_held != 2047 || meeting_held != 255) {
     bad++;
-    printf("failure-handling checks %d of 4095, point-to-point checks %d of 2047\n", failures_held, p2p_held);
+    printf("failure-handling checks %d of 4095, point-to-point checks %d of 2047, meeting checks %d of 255\n", failures_held, p2p_held,
+           meeting_held);
   }
   printf("runs %d bad %d\n", runs, bad);
   return bad != 0;

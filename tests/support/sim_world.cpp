@@ -10,6 +10,7 @@
 
 #include "sim_backend.hpp"
 #include "engine.hpp"
+#include "rendezvous.hpp"
 #include "world.hpp"
 
 using namespace ibcomm_hip;
@@ -28,7 +29,9 @@ struct sim_report {
   char first_race[256];
 };
 
-// threaded = 0: one thread steps all ranks (RunWorld); 1: one thread per rank (AllreduceBlocking).
+// threaded = 0: one thread steps all ranks (RunWorld); 1: one thread per rank, each running its own
+// engine (AllreduceBlocking); 2: one thread per rank, the calls meet and the last to arrive steps all
+// ranks (Rendezvous, what the library's blocking per-rank entry points do).
 // repeats > 1 runs the same collective again on the same communicators (event/slot reuse).
 int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,
                         int max_fuse, int landing, unsigned seed, int threaded, int repeats, sim_report* rep) {
@@ -46,6 +49,7 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
     comms.back()->set_landing(landing);
     raw.push_back(comms.back().get());
   }
+  Rendezvous meet(world);
   for (int k = 0; k < repeats && rc == kOk; k++) {
     if (!threaded) {
       rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, true);
@@ -56,7 +60,28 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
       std::vector<std::thread> th;
       for (int r = 0; r < world; r++) {
         th.emplace_back([&, r]() {
-          rcs[r] = raw[r]->AllreduceBlocking(algo, dtype, sendbufs[r], recvbufs[r], len);
+          if (threaded == 2) {
+            RankCall call;
+            call.comm = raw[r];
+            call.algo = algo;
+            call.dtype = dtype;
+            call.sendbuf = sendbufs[r];
+            call.recvbuf = recvbufs[r];
+            call.len = len;
+            rcs[r] = meet.Arrive(r, call, 60.0, &fabric, [&](const RankCall* calls) {
+              std::vector<Communicator<SimBackend>*> cs(world);
+              std::vector<const void*> sp(world);
+              std::vector<void*> rp(world);
+              for (int i = 0; i < world; i++) {
+                cs[i] = static_cast<Communicator<SimBackend>*>(calls[i].comm);
+                sp[i] = calls[i].sendbuf;
+                rp[i] = calls[i].recvbuf;
+              }
+              return RunWorld<SimBackend>(cs.data(), world, calls[0].algo, calls[0].dtype, sp.data(), rp.data(), calls[0].len, true);
+            });
+          } else {
+            rcs[r] = raw[r]->AllreduceBlocking(algo, dtype, sendbufs[r], recvbufs[r], len);
+          }
           if (rcs[r]) msgs[r] = LastErrorBuffer();
         });
       }
@@ -73,7 +98,7 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   std::string first;
   rep->rc = rc;
   rep->nodes = Sim::Get().node_count();
-  rep->races = threaded ? -1 : Sim::Get().CheckRaces(&first);
+  rep->races = threaded == 1 ? -1 : Sim::Get().CheckRaces(&first);
   rep->unrecorded_waits = Sim::Get().unrecorded_waits();
   if (!raw.empty()) rep->rank0 = raw[0]->stats();
   snprintf(rep->first_race, sizeof rep->first_race, "%s", first.c_str());
@@ -186,6 +211,124 @@ int sim_failures(void) {
       if (rc == kOk && out[100] == 3.0f) held |= 512;
       fabric.StopReplay();
     }
+  }
+  return held;
+}
+
+// The meeting of blocking per-rank calls, forced from the host; returns a bit per check that held.
+int sim_rendezvous(void) {
+  Sim::Get().Reset(11);
+  int held = 0;
+  std::vector<float> a(4096, 1.0f), b(4096, 2.0f), c(4096, 4.0f), ra(4096), rb(4096), rc_buf(4096);
+  auto call_of = [](void* comm, int algo, const void* s, void* r, size_t n) {
+    RankCall k;
+    k.comm = comm;
+    k.algo = algo;
+    k.dtype = kF32;
+    k.sendbuf = s;
+    k.recvbuf = r;
+    k.len = n;
+    return k;
+  };
+  Fabric<SimBackend> fabric(3);
+  Communicator<SimBackend> c0(&fabric, 3), c1(&fabric, 3), c2(&fabric, 3);
+  Communicator<SimBackend>* cs[3] = {&c0, &c1, &c2};
+  for (int r = 0; r < 3; r++) {
+    cs[r]->Init();
+    cs[r]->RegisterMyself(r);
+  }
+  Rendezvous meet(3);
+  int drives = 0;
+  auto drive = [&](const RankCall* calls) {
+    drives++;
+    Communicator<SimBackend>* w[3];
+    const void* sp[3];
+    void* rp[3];
+    for (int i = 0; i < 3; i++) {
+      w[i] = static_cast<Communicator<SimBackend>*>(calls[i].comm);
+      sp[i] = calls[i].sendbuf;
+      rp[i] = calls[i].recvbuf;
+    }
+    return RunWorld<SimBackend>(w, 3, calls[0].algo, calls[0].dtype, sp, rp, calls[0].len, true);
+  };
+  {
+    // three ranks meet, five rounds in a row; one thread drives each round, all get its status
+    int r[3] = {-1, -1, -1};
+    bool ok = true;
+    for (int round = 0; round < 5 && ok; round++) {
+      std::thread t1([&]() { r[1] = meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 4096), 30.0, &fabric, drive); });
+      std::thread t2([&]() { r[2] = meet.Arrive(2, call_of(&c2, kRing, c.data(), rc_buf.data(), 4096), 30.0, &fabric, drive); });
+      r[0] = meet.Arrive(0, call_of(&c0, kRing, a.data(), ra.data(), 4096), 30.0, &fabric, drive);
+      t1.join();
+      t2.join();
+      ok = r[0] == kOk && r[1] == kOk && r[2] == kOk && ra[5] == 7.0f && rb[4095] == 7.0f && rc_buf[0] == 7.0f;
+    }
+    if (ok && drives == 5 && meet.rounds() == 5) held |= 1;
+  }
+  {
+    // ranks that disagree about the length are all told so, with the message in each thread's buffer
+    int r[3] = {-1, -1, -1};
+    std::string m1;
+    const int before = drives;
+    std::thread t1([&]() {
+      r[1] = meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 2048), 30.0, &fabric, drive);
+      m1 = LastErrorBuffer();
+    });
+    std::thread t2([&]() { r[2] = meet.Arrive(2, call_of(&c2, kRing, c.data(), rc_buf.data(), 4096), 30.0, &fabric, drive); });
+    r[0] = meet.Arrive(0, call_of(&c0, kRing, a.data(), ra.data(), 4096), 30.0, &fabric, drive);
+    t1.join();
+    t2.join();
+    if (r[0] == kInvalidArgument && r[1] == kInvalidArgument && r[2] == kInvalidArgument && drives == before &&
+        m1.find("rank 1 entered") != std::string::npos)
+      held |= 2;
+  }
+  {
+    // a failure inside the collective (a world the algorithm does not support) reaches every rank, and
+    // the world stays usable: the driver cleans up after itself
+    int r[3] = {-1, -1, -1};
+    std::thread t1([&]() { r[1] = meet.Arrive(1, call_of(&c1, kRabenseifner, b.data(), rb.data(), 4096), 30.0, &fabric, drive); });
+    std::thread t2([&]() { r[2] = meet.Arrive(2, call_of(&c2, kRabenseifner, c.data(), rc_buf.data(), 4096), 30.0, &fabric, drive); });
+    r[0] = meet.Arrive(0, call_of(&c0, kRabenseifner, a.data(), ra.data(), 4096), 30.0, &fabric, drive);
+    t1.join();
+    t2.join();
+    if (r[0] == kNotSupported && r[1] == kNotSupported && r[2] == kNotSupported && !fabric.poisoned() && !c0.active()) held |= 4;
+  }
+  {
+    // the same rank twice in one round is refused
+    std::thread t1([&]() { (void)meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 4096), 0.5, &fabric, drive); });
+    std::this_thread::sleep_for(std::chrono::milliseconds(100));
+    if (meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 4096), 0.5, &fabric, drive) == kNotSupported) held |= 8;
+    t1.join();  // gives up after its 0.5 s and marks the world
+    if (fabric.poisoned()) held |= 16;
+    // an abandoned world refuses further meetings until its owner resets it
+    if (meet.Arrive(0, call_of(&c0, kRing, a.data(), ra.data(), 4096), 0.5, &fabric, drive) == kTransportError &&
+        strstr(LastErrorBuffer(), "abandoned") != nullptr)
+      held |= 32;
+    fabric.Reset();
+  }
+  {
+    // one rank never comes: the first to lose patience (0.3 s) marks the world and the other stops
+    // waiting at once instead of sitting out its own limit (30 s); nothing was driven
+    int r0 = -1, r1 = -1;
+    std::string m1;
+    const int before = drives;
+    const auto t0 = std::chrono::steady_clock::now();
+    std::thread t([&]() { r0 = meet.Arrive(0, call_of(&c0, kRing, a.data(), ra.data(), 4096), 0.3, &fabric, drive); });
+    r1 = meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 4096), 30.0, &fabric, drive);
+    m1 = LastErrorBuffer();
+    t.join();
+    const double took = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (r0 == kTransportError && r1 == kTransportError && took < 5.0 && m1.find("gave up") != std::string::npos && drives == before)
+      held |= 64;
+    fabric.Reset();
+    // after the reset the three meet again
+    int r[3] = {-1, -1, -1};
+    std::thread t1([&]() { r[1] = meet.Arrive(1, call_of(&c1, kRing, b.data(), rb.data(), 4096), 30.0, &fabric, drive); });
+    std::thread t2([&]() { r[2] = meet.Arrive(2, call_of(&c2, kRing, c.data(), rc_buf.data(), 4096), 30.0, &fabric, drive); });
+    r[0] = meet.Arrive(0, call_of(&c0, kRing, a.data(), ra.data(), 4096), 30.0, &fabric, drive);
+    t1.join();
+    t2.join();
+    if (r[0] == kOk && r[1] == kOk && r[2] == kOk && ra[9] == 7.0f) held |= 128;
   }
   return held;
 }

@@ -59,11 +59,42 @@ def test_many_ranks(algo, world_size):
 
 @pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
 def test_one_thread_per_rank_blocking_calls(algo):
-    # the reference's usage: every rank inside its own blocking call at the same time
+    # the reference's usage: every rank inside its own blocking call at the same time.  The calls meet
+    # and the last rank to arrive drives the world: eager on the first call of a shape, recorded on the
+    # second, replayed afterwards.  Six calls per shape on the same buffers with fresh contents, every
+    # one checked against the oracle.
+    with H.World(4) as w:
+        for n, chunk in ((300001, None), (65536, 4096)):
+            send = G.to_device(rand_bufs(4, n, seed=0))
+            recv = [G.poisoned_like(t) for t in send]
+            for k in range(6):
+                host = rand_bufs(4, n, seed=10 * k + 1)
+                for t, h in zip(send, host):
+                    t.copy_(torch.from_numpy(h))
+                for t in recv:
+                    t.view(torch.uint8).fill_(0x55)
+                assert G.run_world(w, algo, send, recv, chunk, threads=True) == 0, H.last_error()
+                orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
+                assert orc == 0
+                for r in range(4):
+                    assert np.array_equal(O.bits(recv[r].cpu().numpy()), O.bits(want[r])), (n, k, r)
+        eager, captured, replayed = w.graph_counters()
+        assert (eager, captured, replayed) == (2, 2, 10), (eager, captured, replayed)
+        # fresh buffers every call (no shape is ever seen twice in a row at the same addresses)
+        for k in range(3):
+            G.check_against_oracle(w, algo, rand_bufs(4, 300001, seed=k), None, threads=True)
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_one_thread_per_rank_each_with_its_own_engine(algo, monkeypatch):
+    # IBCOMM_HIP_RENDEZVOUS=0: the rank threads do not meet; each runs its own engine and the ranks
+    # exchange messages through the loopback as separate processes would
+    monkeypatch.setenv("IBCOMM_HIP_RENDEZVOUS", "0")
     with H.World(4) as w:
         for k in range(3):
             G.check_against_oracle(w, algo, rand_bufs(4, 300001, seed=k), None, threads=True)
         G.check_against_oracle(w, algo, rand_bufs(4, 65536, seed=9), 4096, threads=True)
+        assert w.graph_counters() == (0, 0, 0)
 
 
 @pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
