@@ -41,6 +41,7 @@
 #include <algorithm>
 #include <chrono>
 #include <deque>
+#include <string>
 #include <thread>
 #include <utility>
 #include <vector>
@@ -143,7 +144,10 @@ class Communicator {
     return trace_.Dump(std::string(base ? base : "ibcomm_trace") + "_" + std::to_string(rank_) + ".dat");
   }
 
-  void RegisterMyself(int rank) { rank_ = rank; }  // ibverbs_communicator.cpp:355-357
+  void RegisterMyself(int rank) {  // ibverbs_communicator.cpp:355-357
+    rank_ = rank;
+    plan_cached_ = false;
+  }
   int rank() const { return rank_; }
   int world_size() const { return world_size_; }
   MemoryPool<B>& pool() { return pool_; }
@@ -185,8 +189,18 @@ class Communicator {
     if (!in_place_ && sendbuf_ < recvbuf_ + bytes && recvbuf_ < sendbuf_ + bytes)
       return Fail(kInvalidArgument, "sendbuf and recvbuf overlap partially");
 
-    // IBCOMM_CHUNKSIZE is read on every call (ibverbs_communicator.cpp:619-634).
-    IBCOMM_RETURN_IF_ERROR(BuildPlan(algo, world_size_, rank_, len_elements, es_, getenv("IBCOMM_CHUNKSIZE"), &plan_));
+    // IBCOMM_CHUNKSIZE is read on every call (ibverbs_communicator.cpp:619-634); the plan it leads to
+    // is kept for as long as the call shape stays the same.
+    const char* chunk_env = getenv("IBCOMM_CHUNKSIZE");
+    const std::string chunk_text = chunk_env ? std::string("=") + chunk_env : std::string();
+    if (!(plan_cached_ && plan_.algo == algo && plan_len_ == len_elements && plan_es_ == es_ && plan_chunk_env_ == chunk_text)) {
+      plan_cached_ = false;
+      IBCOMM_RETURN_IF_ERROR(BuildPlan(algo, world_size_, rank_, len_elements, es_, chunk_env, &plan_));
+      plan_len_ = len_elements;
+      plan_es_ = es_;
+      plan_chunk_env_ = chunk_text;
+      plan_cached_ = true;
+    }
     stats_.calls++;
     // Events of the call before last are free again: a peer trails this rank by at most one
     // collective, because finishing a collective needs every peer to have taken part in it.
@@ -729,11 +743,19 @@ class Communicator {
         {
           // One entry per partial sum accepted, whether or not it needs a landing slot of its own.
           TraceScope scope(&trace_, Trace::kIssueRecv);
-          if (!ZeroCopyReceive()) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+          if (!ZeroCopyReceive() && !controller_.TryGetMemory(&p.slot)) {
+            // Every slot is taken by a message waiting in this pass: launch what has been collected,
+            // which hands its landing slots back (their next use is ordered on the device), and go
+            // on with those.  Only a pool whose blocks hold no slot of this size at all grows.
+            IBCOMM_RETURN_IF_ERROR(FlushReduces());
+            IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.slot));
+          }
         }
         // Nobody on this rank reads a partial sum that is only forwarded: it is produced where the
-        // next rank will fetch it.
-        if (landing_ == kLandStaged && plan_.forward_only[p.op] >= 0) IBCOMM_RETURN_IF_ERROR(controller_.getMemory(&p.stage));
+        // next rank will fetch it, in a staging slot.  Staging slots come back when the next rank has
+        // taken the message, which this rank cannot hurry; when none is left the sum goes to recvbuf
+        // and is forwarded from there, as every sum is in the `direct` mode.
+        if (landing_ == kLandStaged && plan_.forward_only[p.op] >= 0) (void)controller_.TryGetMemory(&p.stage);
         if (!pending_reduce_.empty()) p.joins = ReduceJoins(pending_reduce_.back(), p, pending_reduce_.back().joins);
         if (p.joins == 0 && reduce_runs_ == kMaxSegments) IBCOMM_RETURN_IF_ERROR(FlushReduces());
         if (p.joins == 0) reduce_runs_++;
@@ -748,57 +770,55 @@ class Communicator {
     return kOk;
   }
 
-  // Finished chunks: recvbuf[c] <- message.
+  // Issues the copies a pass has collected on stream s: one copy-kernel launch for all of them, or, in
+  // the `memcpy` mode, one device copy per segment (a run of chunks that follow one another at both
+  // ends).  *issued counts launches or copies.
+  int IssueCopies(const SegmentBatch& batch, Stream s, int role, uint64_t* issued) {
+    if (batch.count == 0) return kOk;
+    if (landing_ != kLandMemcpy) {
+      IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
+      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, role));
+      IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
+      (*issued)++;
+      return kOk;
+    }
+    for (int i = 0; i < batch.count; i++) {
+      const Segment& seg = batch.seg[i];
+      IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
+      IBCOMM_RETURN_IF_ERROR(B::CopyAsync(seg.dst, seg.a, seg.n * es_, s));
+      IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
+      (*issued)++;
+    }
+    return kOk;
+  }
+
+  // Finished chunks: recvbuf[c] <- message.  All copies of a pass go to one stream and share one
+  // event and one batch of completions (a stream, an event and a cross-stream wait per message cost
+  // the host twice what an 8 MiB copy takes on the device).
   int FlushGathers() {
     if (pending_gather_.empty()) return kOk;
     waited_.clear();
     TraceScope scope(&trace_, Trace::kIssueCopyKernel);
-    if (landing_ != kLandMemcpy) {
-      Stream s;
-      IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
-      SegmentBatch batch;
-      batch.count = 0;
-      for (const PendingRecv& p : pending_gather_) {
-        const int c = plan_.recvs[p.op].chunk;
-        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
-        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
-        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
-        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
-        AppendSegment(&batch, Segment{RecvPtr(c), p.msg.src, nullptr, ChunkElems(c)}, p.joins);
-        stats_.gather_bytes += ChunkBytes(c);
-      }
-      IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 2));
-      IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
-      stats_.gather_copies++;
-      OpState done;
-      IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
-      CompleteAll(pending_gather_, done);
-      for (const PendingRecv& p : pending_gather_) {
-        recv_done_[p.op] = done;
-        chunk_last_[plan_.recvs[p.op].chunk] = done;
-      }
-    } else {
-      for (const PendingRecv& p : pending_gather_) {
-        const RecvOp& r = plan_.recvs[p.op];
-        const int c = r.chunk;
-        Stream s;
-        IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
-        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
-        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
-        IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
-        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
-        IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(RecvPtr(c), p.msg.src, ChunkBytes(c), s));
-        IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
-        stats_.gather_copies++;
-        stats_.gather_bytes += ChunkBytes(c);
-        OpState done;
-        IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, done.event, true, done.stream);
-        recv_done_[p.op] = done;
-        chunk_last_[c] = done;
-      }
+    Stream s;
+    IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+    SegmentBatch batch;
+    batch.count = 0;
+    for (const PendingRecv& p : pending_gather_) {
+      const int c = plan_.recvs[p.op].chunk;
+      IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, p.msg));
+      IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_pulled_[c]));
+      IBCOMM_RETURN_IF_ERROR(WaitOn(s, chunk_last_[c]));
+      IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, s));
+      AppendSegment(&batch, Segment{RecvPtr(c), p.msg.src, nullptr, ChunkElems(c)}, p.joins);
+      stats_.gather_bytes += ChunkBytes(c);
+    }
+    IBCOMM_RETURN_IF_ERROR(IssueCopies(batch, s, 2, &stats_.gather_copies));
+    OpState done;
+    IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+    CompleteAll(pending_gather_, done);
+    for (const PendingRecv& p : pending_gather_) {
+      recv_done_[p.op] = done;
+      chunk_last_[plan_.recvs[p.op].chunk] = done;
     }
     pending_gather_.clear();
     gather_runs_ = 0;
@@ -811,66 +831,40 @@ class Communicator {
     waited_.clear();
     const size_t n = pending_reduce_.size();
     Stream s{};
-    std::vector<OpState> landed(n);
 
     trace_.Mark(Trace::kIssueCopyKernel);
-    if (landing_ == kLandMemcpy) {
+    IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
+    for (size_t i = 0; i < n; i++) {
+      IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, pending_reduce_[i].msg));
+      IBCOMM_RETURN_IF_ERROR(RecordPayload(pending_reduce_[i].msg, s));
+    }
+    if (!ZeroCopyReceive()) {
+      // Land every message in its pool slot, on the stream of the reduction that follows: one event
+      // and one batch of completions for the pass.
+      SegmentBatch copy;
+      copy.count = 0;
       for (size_t i = 0; i < n; i++) {
         PendingRecv& p = pending_reduce_[i];
-        const RecvOp& r = plan_.recvs[p.op];
-        Stream si;
-        IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&si));
-        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(si, p.msg));
-        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(si, p.slot));
-        IBCOMM_RETURN_IF_ERROR(RecordPayload(p.msg, si));
-        IBCOMM_RETURN_IF_ERROR(SpanBegin(si, Trace::kDeviceCopy));
-        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(p.slot->LandingFor(RecvPtr(r.chunk)), p.msg.src, ChunkBytes(r.chunk), si));
-        IBCOMM_RETURN_IF_ERROR(SpanEnd(si));
-        stats_.landing_copies++;
-        stats_.landing_bytes += ChunkBytes(r.chunk);
-        IBCOMM_RETURN_IF_ERROR(RecordEvent(si, &landed[i]));
-        fabric_->Complete(rank_, r.peer, p.msg.ticket, landed[i].event, true, landed[i].stream);
-      }
-      s = landed[0].stream;
-      for (size_t i = 1; i < n; i++) IBCOMM_RETURN_IF_ERROR(WaitOn(s, landed[i]));
-    } else {
-      IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
-      for (size_t i = 0; i < n; i++) {
-        IBCOMM_RETURN_IF_ERROR(WaitOnMessage(s, pending_reduce_[i].msg));
-        IBCOMM_RETURN_IF_ERROR(RecordPayload(pending_reduce_[i].msg, s));
-      }
-      if (landing_ == kLandKernel) {
-        SegmentBatch copy;
-        copy.count = 0;
-        for (size_t i = 0; i < n; i++) {
-          PendingRecv& p = pending_reduce_[i];
-          const int c = plan_.recvs[p.op].chunk;
-          IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.slot));
-          // the slots of a run continue one another; the sources may or may not
-          int joins = 0;
-          if (p.joins != 0 && copy.count > 0) {
-            const PendingRecv& q = pending_reduce_[i - 1];
-            const int qc = plan_.recvs[q.op].chunk;
-            if (Adjacent(q.msg.src, ChunkBytes(qc), p.msg.src, ChunkBytes(c)) == p.joins) joins = p.joins;
-          }
-          if (joins == 0 && copy.count == kMaxSegments) {
-            IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-            IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
-            IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
-            stats_.landing_copies++;
-            copy.count = 0;
-          }
-          AppendSegment(&copy, Segment{p.slot->LandingFor(RecvPtr(c)), p.msg.src, nullptr, ChunkElems(c)}, joins);
-          stats_.landing_bytes += ChunkBytes(c);
+        const int c = plan_.recvs[p.op].chunk;
+        IBCOMM_RETURN_IF_ERROR(WaitOnSlot(s, p.slot));
+        // the slots of a run continue one another; the sources may or may not
+        int joins = 0;
+        if (p.joins != 0 && copy.count > 0) {
+          const PendingRecv& q = pending_reduce_[i - 1];
+          const int qc = plan_.recvs[q.op].chunk;
+          if (Adjacent(q.msg.src, ChunkBytes(qc), p.msg.src, ChunkBytes(c)) == p.joins) joins = p.joins;
         }
-        IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-        IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(copy, dtype_, s, 1));
-        IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
-        stats_.landing_copies++;
-        OpState done;
-        IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
-        CompleteAll(pending_reduce_, done);
+        if (joins == 0 && copy.count == kMaxSegments) {
+          IBCOMM_RETURN_IF_ERROR(IssueCopies(copy, s, 1, &stats_.landing_copies));
+          copy.count = 0;
+        }
+        AppendSegment(&copy, Segment{p.slot->LandingFor(RecvPtr(c)), p.msg.src, nullptr, ChunkElems(c)}, joins);
+        stats_.landing_bytes += ChunkBytes(c);
       }
+      IBCOMM_RETURN_IF_ERROR(IssueCopies(copy, s, 1, &stats_.landing_copies));
+      OpState done;
+      IBCOMM_RETURN_IF_ERROR(RecordEvent(s, &done));
+      CompleteAll(pending_reduce_, done);
     }
 
     trace_.Mark(Trace::kIssueCopyKernel);
@@ -972,6 +966,9 @@ class Communicator {
   bool finished_ = false;
   bool in_place_ = false;
   Plan plan_;
+  bool plan_cached_ = false;       // plan_ is the plan of (plan_.algo, plan_len_, plan_es_, plan_chunk_env_) for this rank
+  size_t plan_len_ = 0, plan_es_ = 0;
+  std::string plan_chunk_env_;     // "" = IBCOMM_CHUNKSIZE unset, else "=" + its text
   int dtype_ = kF32;
   size_t es_ = 4;
   const char* sendbuf_ = nullptr;

@@ -12,9 +12,15 @@
 //     *enqueued*, together with the event that marks that kernel's completion;
 //     the next user of the slot orders itself after that event on the device.
 //     The host never waits for a slot, so a handful of slots sustain the whole
-//     pipeline and the pool does not grow with the buffer; returned slots are
-//     reused before untouched ones, so those few slots are also all the memory
-//     a collective's staging ever writes;
+//     pipeline; returned slots are reused before untouched ones, so those few
+//     slots are also all the memory a collective's staging ever writes.  The
+//     engine never grows the pool in the middle of a collective as long as its
+//     blocks hold one slot: when every slot is taken it launches what it has
+//     collected (which hands the landing slots back) or, for send staging,
+//     leaves the partial sum in recvbuf; getMemory() itself still grows the
+//     pool on exhaustion, as the reference's does (memory_pool.h:229-231);
+//   * slots are carved on demand, so a block of tiny chunks costs nothing for
+//     the slots nobody asks for and no cap on their number is needed;
 //   * each slot keeps 16 spare bytes so that a message can land at the same
 //     16-byte phase as the recvbuf range it will be added to, which keeps the
 //     kernel's body on dwordx4 accesses for odd chunk offsets;
@@ -63,7 +69,10 @@ class MemoryController {
   ~MemoryController() { Release(); }
 
   bool active() const { return pool_ != nullptr; }
-  size_t slot_count() const { return slots_.size(); }
+  // Slots the pool's blocks hold at this chunk size, handed out yet or not.
+  size_t slot_count() const { return capacity_; }
+  // Slots that can be handed out without growing the pool.
+  size_t available() const { return vacant_.size() + (capacity_ - carved_); }
   int held() const { return held_; }
   int high_water() const { return high_water_; }
 
@@ -74,6 +83,8 @@ class MemoryController {
   // step's stores into it run measurably faster than stores that walk through the whole block
   // (config 2: 205 -> 196 us per rank schedule).
   int getMemory(Memory<B>** out);
+  // The same without growth: false (and *out untouched) when every slot is taken.
+  bool TryGetMemory(Memory<B>** out);
   // FIFO return (memory_pool.h:238-242); `after` completes when the slot's contents are dead.
   void returnMemory(Memory<B>* m, typename B::Event after, typename B::Stream stream) {
     m->free_event = after;
@@ -90,14 +101,25 @@ class MemoryController {
 
  private:
   friend class MemoryPool<B>;
-  void Carve(char* block, size_t block_bytes);
+  struct Block {
+    char* base;
+    size_t slots;  // block bytes / stride
+  };
+  void AddBlock(char* block, size_t block_bytes) {
+    blocks_.push_back(Block{block, block_bytes / stride_});
+    capacity_ += blocks_.back().slots;
+  }
+  Memory<B>* CarveNext();
 
   MemoryPool<B>* pool_ = nullptr;
   size_t stride_ = 0;
   bool descending_ = false;
-  std::vector<std::unique_ptr<Memory<B>>> slots_;
+  std::vector<Block> blocks_;      // the pool's blocks as this chunk size divides them
+  size_t capacity_ = 0;            // slots in all blocks
+  size_t carved_ = 0;              // of which handed out at least once, block after block, in the hand-out direction
+  size_t carve_block_ = 0, carve_slot_ = 0;  // the next untouched slot
+  std::vector<std::unique_ptr<Memory<B>>> slots_;  // one object per slot handed out so far
   std::deque<Memory<B>*> vacant_;  // returned, oldest first
-  std::deque<Memory<B>*> fresh_;   // never handed out, in address order of the hand-out direction
   int held_ = 0;
   int high_water_ = 0;
 };
@@ -142,10 +164,11 @@ class MemoryPool {
     c->descending_ = descending;
     c->slots_.clear();
     c->vacant_.clear();
-    c->fresh_.clear();
+    c->blocks_.clear();
+    c->capacity_ = c->carved_ = c->carve_block_ = c->carve_slot_ = 0;
     c->held_ = 0;
     c->high_water_ = 0;
-    for (auto& b : blocks_) c->Carve(b.first, b.second);
+    for (auto& b : blocks_) c->AddBlock(b.first, b.second);
     return kOk;
   }
 
@@ -238,40 +261,53 @@ class MemoryPool {
   bool has_override_ = false;
 };
 
+// The next slot nobody has used yet: blocks in the order they were allocated, inside a block from the
+// lowest address upwards or, descending, from the highest downwards.
 template <class B>
-void MemoryController<B>::Carve(char* block, size_t block_bytes) {
-  // Slots are reused first-in first-out and a pass holds at most one launch's worth of them, so
-  // beyond a few hundred more slots buy nothing; tiny chunks would otherwise yield millions.
-  constexpr size_t kMaxSlotsPerBlock = 1024;
-  size_t count = block_bytes / stride_;
-  if (count > kMaxSlotsPerBlock) count = kMaxSlotsPerBlock;
-  for (size_t k = 0; k < count; k++) {
-    const size_t i = descending_ ? count - 1 - k : k;
-    slots_.emplace_back(new Memory<B>());
-    Memory<B>* m = slots_.back().get();
-    m->base = block + i * stride_;
-    m->capacity = stride_;
-    fresh_.push_back(m);
+Memory<B>* MemoryController<B>::CarveNext() {
+  while (carve_block_ < blocks_.size() && carve_slot_ == blocks_[carve_block_].slots) {
+    carve_block_++;
+    carve_slot_ = 0;
   }
+  if (carve_block_ == blocks_.size()) return nullptr;
+  const Block& b = blocks_[carve_block_];
+  const size_t i = descending_ ? b.slots - 1 - carve_slot_ : carve_slot_;
+  carve_slot_++;
+  carved_++;
+  slots_.emplace_back(new Memory<B>());
+  Memory<B>* m = slots_.back().get();
+  m->base = b.base + i * stride_;
+  m->capacity = stride_;
+  return m;
+}
+
+template <class B>
+bool MemoryController<B>::TryGetMemory(Memory<B>** out) {
+  if (!pool_) return false;
+  Memory<B>* m = nullptr;
+  if (!vacant_.empty()) {
+    m = vacant_.front();
+    vacant_.pop_front();
+  } else {
+    m = CarveNext();
+  }
+  if (!m) return false;
+  held_++;
+  if (held_ > high_water_) high_water_ = held_;
+  *out = m;
+  return true;
 }
 
 template <class B>
 int MemoryController<B>::getMemory(Memory<B>** out) {
   if (!pool_) return Fail(kInvalidArgument, "MemoryController is not attached to a pool");
-  if (vacant_.empty() && fresh_.empty()) {
-    size_t bytes = pool_->block_bytes();
-    if (bytes < 2 * stride_) bytes = 2 * stride_;
-    char* block = nullptr;
-    IBCOMM_RETURN_IF_ERROR(pool_->AllocateBlock(bytes, &block));
-    Carve(block, bytes);
-  }
-  std::deque<Memory<B>*>& from = vacant_.empty() ? fresh_ : vacant_;
-  Memory<B>* m = from.front();
-  from.pop_front();
-  held_++;
-  if (held_ > high_water_) high_water_ = held_;
-  *out = m;
-  return kOk;
+  if (TryGetMemory(out)) return kOk;
+  size_t bytes = pool_->block_bytes();
+  if (bytes < 2 * stride_) bytes = 2 * stride_;
+  char* block = nullptr;
+  IBCOMM_RETURN_IF_ERROR(pool_->AllocateBlock(bytes, &block));
+  AddBlock(block, bytes);
+  return TryGetMemory(out) ? kOk : Fail(kDeviceError, "a new pool block of %zu bytes holds no slot of %zu", bytes, stride_);
 }
 
 template <class B>
@@ -279,7 +315,8 @@ void MemoryController<B>::Release() {
   if (!pool_) return;
   slots_.clear();
   vacant_.clear();
-  fresh_.clear();
+  blocks_.clear();
+  capacity_ = carved_ = carve_block_ = carve_slot_ = 0;
   pool_->CompleteMemoryController();
   pool_ = nullptr;
 }

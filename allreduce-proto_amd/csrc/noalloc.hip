@@ -122,8 +122,11 @@ extern "C" int ibcomm_hip_world_allreduce_noalloc(int world_size, int algo, int 
   const size_t es = DTypeSize(dtype);
   if (es == 0) return Fail(kInvalidArgument, "unsupported element type %d", dtype);
 
-  // Staging the call can need at most: every rank holding two slots per chunk of the buffer.
-  // Checked before anything is enqueued, so a refused call leaves the stream untouched.
+  // Staging the call can use at most: every rank holding two slots per chunk of the buffer (the
+  // sums it has produced for the next rank and those it is producing).  Each rank's pool gets one
+  // block of exactly that size out of the array below, before anything is enqueued, and the engine
+  // never asks a pool that holds a slot for another block; so a call is either refused here, with
+  // the stream untouched, or runs to its end.
   size_t block_bytes = 0;
   if (world_size > 1) {
     std::vector<Range> ranges;

@@ -21,7 +21,8 @@ def rand_bufs(world, n, seed=0, dtype=np.float32):
     return [(np.random.default_rng(seed + r).standard_normal(n) * 3).astype(dtype) for r in range(world)]
 
 
-def check(algo, bufs, chunk=None, **kw):
+def check(algo, bufs, chunk=None, unchecked_ok=False, **kw):
+    """unchecked_ok: the run may be too large for the simulator's race check (races == -1)."""
     rc, recv, rep = S.allreduce(algo, bufs, chunk, **kw)
     assert rc == 0, rep.error.decode()
     orc, want, _ = O.allreduce(ORACLE_ALGO[algo], bufs, chunk)
@@ -30,7 +31,7 @@ def check(algo, bufs, chunk=None, **kw):
         assert np.array_equal(O.bits(recv[r]), O.bits(want[r])), "rank %d differs from the oracle" % r
     assert rep.unrecorded_waits == 0
     if kw.get("threaded", 0) != 1:  # with one engine per thread the graph of device work is not checked for races
-        assert rep.races == 0, rep.first_race.decode()
+        assert rep.races == 0 or (unchecked_ok and rep.races == -1), rep.first_race.decode()
     return rep
 
 
@@ -72,6 +73,25 @@ def test_tiny_pool_forces_slot_reuse(algo, world):
     # a pool smaller than one chunk grows instead of failing
     rep = check(algo, bufs, 1024, max_fuse=4, landing=1, pool_bytes=64, seed=9)
     assert rep.rank0.pool_blocks >= 2
+
+
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+@pytest.mark.parametrize("pool_bytes", [1 << 16, 64 << 20])
+def test_thousands_of_chunks_per_step_do_not_grow_the_pool(landing, pool_bytes):
+    # 4 ranks x 1 Mi fp32 in 256-byte chunks: 4,096 chunks per ring step.  A rank collects every message
+    # that is there before it launches, and each of them wants a landing or a staging slot: with slots
+    # for 256 chunks (64 KiB block) or 262,144 (64 MiB) the collective must get by on the one block the
+    # pool was created with -- launching early, or leaving partial sums in recvbuf -- and stay bit-exact.
+    bufs = rand_bufs(4, 1 << 20, seed=21)
+    big = landing == 0  # one device copy per message: some 200,000 operations
+    rep = check(RING, bufs, 256, unchecked_ok=big, max_fuse=64, landing=landing, pool_bytes=pool_bytes, seed=landing)
+    assert rep.rank0.pool_blocks == 1 and rep.rank0.pool_bytes == pool_bytes
+    assert rep.rank0.slot_count == pool_bytes // 256
+    assert rep.rank0.slots_high_water <= rep.rank0.slot_count
+    if landing == 3:
+        assert rep.rank0.slots_high_water == min(pool_bytes // 256, 2 * 4096)
+    rep = check(RABEN, bufs, 256, unchecked_ok=big, max_fuse=64, landing=landing, pool_bytes=pool_bytes, seed=landing)
+    assert rep.rank0.pool_blocks == 1
 
 
 @pytest.mark.parametrize("algo,world", [(RING, 2), (RING, 4), (RABEN, 2), (RABEN, 8)])
@@ -183,7 +203,10 @@ def test_contiguous_chunks_merge_into_one_kernel_segment(landing):
     st = check(RING, bufs, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
     assert st.reduce_segments == (world - 1) * q
     assert st.reduce_launches == world - 1 and st.reduce_kernel_segments == world - 1
-    assert st.gather_copies == (world - 1 if landing else (world - 1) * q)
+    # the chunks of a gather step merge as well: one copy-kernel launch, or (landing 0) one device copy, per step
+    assert st.gather_copies == world - 1
+    if landing == 0:
+        assert st.landing_copies == world - 1  # a step's messages land in adjacent slots through one device copy
     # Rabenseifner rank 0 of 4: two halving steps over 2 and 1 groups
     st = check(RABEN, bufs, chunk, max_fuse=64, landing=landing, pool_bytes=1 << 20).rank0
     # (staged: the half of the first window that is passed on in the second step goes to send staging,

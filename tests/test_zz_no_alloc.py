@@ -2,7 +2,9 @@
 a variant of, ibcomm_hip_world_allreduce: same inputs through the C ABI, outputs compared bit for bit, on
 two calls in a row of which the second is smaller (it finds the first call's staging data in the
 library's built-in array).  Also against the CPU oracle, that free device memory does not move across
-the calls, and that a size beyond the built-in array is refused before anything is enqueued."""
+the calls, that a size beyond the built-in array is refused before anything is enqueued, that the largest
+accepted size with thousands of chunks per rank completes, and that the call can be recorded into a HIP
+graph and replayed."""
 import numpy as np
 import pytest
 
@@ -103,3 +105,58 @@ def test_sizes_beyond_the_built_in_array_are_refused():
     rc = H.world_allreduce_noalloc(3, H.RABENSEIFNER, H.F32, [t.data_ptr() for t in three], [t.data_ptr() for t in out], 64, None)
     torch.cuda.synchronize()
     assert rc == H.NOT_SUPPORTED  # Rabenseifner on a world that is not a power of two
+
+
+def test_the_largest_accepted_call_with_thousands_of_chunks_completes():
+    # 4 ranks x 1 Mi fp32 in 256-byte chunks: 16,384 chunks, 4,096 per ring step; the refusal rule
+    # (ranks x 2 x chunks x 512 bytes) comes to exactly the 64 MiB the array holds, so the call is accepted
+    # -- and then has to finish: every rank's one block must hold the slots the rule promised.
+    world, n, chunk = 4, 1 << 20, 256
+    host = bufs(world, n, 31)
+    send = G.to_device(host)
+    for algo in (H.RING, H.RABENSEIFNER):
+        rc, got = no_alloc(world, algo, send, chunk)
+        assert rc == 0, H.last_error()
+        orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host, chunk)
+        assert orc == 0
+        for r in range(world):
+            assert np.array_equal(O.bits(got[r].cpu().numpy()), O.bits(want[r])), (algo, r)
+    # one element more per rank and the rule refuses, with recvbufs untouched
+    send = G.to_device(bufs(world, n + 64, 32))
+    recv = [torch.full((n + 64,), 7.0, device="cuda") for _ in range(world)]
+    with G.env(IBCOMM_CHUNKSIZE=chunk):
+        rc = H.world_allreduce_noalloc(world, H.RING, H.F32, [t.data_ptr() for t in send], [t.data_ptr() for t in recv], n + 64, None)
+    torch.cuda.synchronize()
+    assert rc == H.INVALID_ARGUMENT and "built-in" in H.last_error()
+    assert all(bool((t == 7.0).all()) for t in recv)
+
+
+@pytest.mark.parametrize("algo", [H.RING, H.RABENSEIFNER])
+def test_recorded_into_a_hip_graph_and_replayed(algo):
+    # a caller under stream capture cannot allocate: the call must record as kernel launches only.  The
+    # first call on the device (which looks up the built-in array) is made outside the capture; the
+    # graph is replayed three times with fresh inputs and other device work in between, and every
+    # replay is checked against the eager result of the allocating entry point.
+    world, n, chunk = 4, 100003, None
+    send = G.to_device(bufs(world, n, 41))
+    recv = [G.poisoned_like(t) for t in send]
+    sp, rp = [t.data_ptr() for t in send], [t.data_ptr() for t in recv]
+    assert H.world_allreduce_noalloc(world, algo, H.F32, sp, rp, n, None) == 0, H.last_error()
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s, capture_error_mode="thread_local"):
+        rc = H.world_allreduce_noalloc(world, algo, H.F32, sp, rp, n, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, H.last_error()
+    for k in range(3):
+        host = bufs(world, n, 50 + k)
+        for t, h in zip(send, host):
+            t.copy_(torch.from_numpy(h))
+        for t in recv:
+            t.view(torch.uint8).fill_(0x55)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = existing_entry_point(world, algo, send, chunk)
+        for r in range(world):
+            assert G.bits_equal(recv[r], want[r]), (k, r)
