@@ -96,9 +96,18 @@ struct HipBackend {
     return kOk;
   }
   // `role` says what the launch is for (0 = reduction, 1 = landing copy into a pool slot,
-  // 2 = gather into recvbuf); the kernels are the same for all three.
-  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0) {
-    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, s));
+  // 2 = gather into recvbuf); the kernels are the same for all three.  With timers the kernel leaves
+  // its own begin and end times in them; a batch without elements launches nothing, and then the
+  // timers are recorded on the stream so that they still hold a (zero-length) span.
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0, Timer start = nullptr, Timer stop = nullptr) {
+    bool empty = true;
+    for (int i = 0; i < batch.count; i++) empty = empty && batch.seg[i].n == 0;
+    if (empty && start && stop) {
+      IBCOMM_HIP_CHECK(hipEventRecord(start, s));
+      IBCOMM_HIP_CHECK(hipEventRecord(stop, s));
+      return kOk;
+    }
+    IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, s, start, stop));
     return kOk;
   }
 };

@@ -699,6 +699,8 @@ int ibcomm_hip_comm_set_timer_base(ibcomm_hip_comm* comm) {
 
 int ibcomm_hip_comm_set_trace(ibcomm_hip_comm* comm, int enabled) {
   if (!comm) return Fail(kInvalidArgument, "comm is null");
+  // switching the trace on starts a fresh recording
+  if (enabled != 0 && !comm->comm.trace().enabled()) comm->comm.trace().Clear();
   comm->comm.trace().Enable(enabled != 0);
   return kOk;
 }

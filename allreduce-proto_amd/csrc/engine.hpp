@@ -600,6 +600,19 @@ class Communicator {
     if (!DeviceTiming()) return kOk;
     return B::TimerRecord(spans_.back().stop, s);
   }
+  // A kernel launch takes the span's two timers itself and leaves its own begin and end times in
+  // them: the span is then the kernel's duration, without the few microseconds it costs the
+  // device to process a marker before and after it.
+  int LaunchTimed(const SegmentBatch& batch, Stream s, int role, Trace::DeviceCategory category) {
+    if (!DeviceTiming()) return B::LaunchSegments(batch, dtype_, s, role);
+    DeviceSpan span;
+    span.category = category;
+    IBCOMM_RETURN_IF_ERROR(NextTimer(&span.start));
+    IBCOMM_RETURN_IF_ERROR(NextTimer(&span.stop));
+    if (spans_.empty()) span_origin_ms_ = trace_.NowMs();
+    spans_.push_back(span);
+    return B::LaunchSegments(batch, dtype_, s, role, span.start, span.stop);
+  }
   // After the streams have drained: turn the timer pairs of this call into trace entries.
   int ResolveDeviceSpans() {
     for (const DeviceSpan& span : spans_) {
@@ -776,9 +789,7 @@ class Communicator {
   int IssueCopies(const SegmentBatch& batch, Stream s, int role, uint64_t* issued) {
     if (batch.count == 0) return kOk;
     if (landing_ != kLandMemcpy) {
-      IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-      IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, role));
-      IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
+      IBCOMM_RETURN_IF_ERROR(LaunchTimed(batch, s, role, Trace::kDeviceCopy));
       (*issued)++;
       return kOk;
     }
@@ -883,9 +894,7 @@ class Communicator {
       AppendSegment(&batch, Segment{ResultOf(p), IncomingOf(p), OwnOf(p), ChunkElems(c)}, p.joins);
       stats_.reduce_elements += ChunkElems(c);
     }
-    IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceReduce));
-    IBCOMM_RETURN_IF_ERROR(B::LaunchSegments(batch, dtype_, s, 0));
-    IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
+    IBCOMM_RETURN_IF_ERROR(LaunchTimed(batch, s, 0, Trace::kDeviceReduce));
     stats_.reduce_launches++;
     stats_.reduce_segments += n;
     stats_.reduce_kernel_segments += batch.count;

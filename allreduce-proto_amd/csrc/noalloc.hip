@@ -106,7 +106,7 @@ struct StaticBackend {
     IBCOMM_HIP_CHECK(LaunchCopy(dst, src, bytes / 4, kI32, s));
     return kOk;
   }
-  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0) {
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int /*role*/ = 0, Timer = 0, Timer = 0) {
     IBCOMM_HIP_CHECK(::ibcomm_hip::LaunchSegments(batch, dtype, s));
     return kOk;
   }

@@ -1,6 +1,8 @@
 // gfx950 streaming add / copy kernels.  See reduce_kernels.hpp for the contract.
 #include "reduce_kernels.hpp"
 
+#include <hip/hip_ext.h>
+
 namespace ibcomm_hip {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -10,15 +12,21 @@ typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
 
 // Cache policy of the streaming accesses.  Loads carry the non-temporal hint: nothing is read
 // twice, so neither the L2 nor the memory-side cache should keep the lines.  Stores of the aligned
-// kernel carry the system coherence scope instead (sc1): they are written through to the memory
-// side, where the 256 MB cache in front of HBM absorbs them and writes them back in longer runs
-// than the kernel's own interleaving of two reads and one write would give the DRAM; and a
-// destination that is written again soon (a rank's few staging slots) is still there.  Measured on
-// MI355X against non-temporal stores: a ring step of 32 MiB per operand into a 64 MiB staging ring
-// 7 % faster, copies of 32 to 64 MiB 3 to 4 % faster, nothing gained once a launch writes more
-// than about half that cache, where non-temporal stores are 1 to 2 % ahead; the host picks by the
-// bytes a launch writes.  The builtin offers no such store, hence the one instruction of inline
-// assembly; the compiler still schedules everything around it.
+// kernel carry the sc1 bit instead.  In the memory model of the gfx940 family sc1 alone marks an
+// access as agent (device) scope; system scope is sc0 sc1.  The device has eight L2s, one per die, so
+// an agent-scope store cannot stay behind in the L2 of the die that issued it; it has to reach
+// the level all dies share, which is where the 256 MB cache in front of HBM sits.  That much is
+// the model; what is measured on MI355X, against non-temporal stores: a ring step of 32 MiB per
+// operand whose results cycle through a 64 MiB staging region is 7 % faster (15.3 against 16.6 us),
+// copies of 32 to 64 MiB are 3 to 4 % faster, sc0 sc1 (system scope) performs like sc1, and once a
+// launch writes more than about half of that cache nothing is gained and non-temporal stores are 1
+// to 2 % ahead; the host picks by the bytes a launch writes.  The explanation offered for the gain
+// (the stores are absorbed by the memory-side cache, which writes back in longer runs than the
+// kernel's interleaving of two reads and one write gives the DRAM, and a destination written
+// again soon is still there) fits the dependence on the size of the destination but has not been
+// confirmed with a counter that separates cache hits from DRAM writes.  The builtin offers no such
+// store, hence the one instruction of inline assembly; the compiler still schedules everything
+// around it.
 template <typename V>
 __device__ __forceinline__ void StoreWriteThrough(V* p, V v) {
   static_assert(sizeof(V) == 16, "one 16-byte vector");
@@ -31,7 +39,7 @@ template <int N>
 struct KernelSegments {
   Segment seg[N];
   uint32_t die_local_tiles;
-  uint32_t write_through;  // stores carry the system scope (see StoreWriteThrough) instead of the non-temporal hint
+  uint32_t write_through;  // stores carry sc1, the agent-scope bit (see StoreWriteThrough), instead of the non-temporal hint
 };
 
 template <int N>
@@ -159,8 +167,18 @@ __global__ __launch_bounds__(THREADS) void AlignedOneSegmentKernel(V* dst, const
 
 namespace {
 
+// With `start` / `stop` set the launch goes through the extended call, which makes the two events
+// carry the kernel's own begin and end timestamps (what a profiler reports for the dispatch) instead
+// of the times at which markers before and after it were processed.
+template <typename... Params, typename... Args>
+void Launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, hipEvent_t start, hipEvent_t stop, Args... args) {
+  if (start || stop) hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, start, stop, 0, args...);
+  else hipLaunchKernelGGL(kernel, grid, block, 0, stream, args...);
+}
+
 template <typename V, int PER_VEC, int THREADS>
-hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream) {
+hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream, hipEvent_t e0,
+                            hipEvent_t e1) {
   const uint64_t blocks = (max_nvec + THREADS - 1) / THREADS;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(batch.count));
@@ -170,27 +188,28 @@ hipError_t LaunchAlignedOne(const SegmentBatch& batch, uint64_t max_nvec, bool a
   if (batch.count == 1) {
     const Segment& s = batch.seg[0];
     if (add)
-      hipLaunchKernelGGL((AlignedOneSegmentKernel<V, THREADS, true>), grid, dim3(THREADS), 0, stream, static_cast<V*>(s.dst),
-                         static_cast<const V*>(s.a), static_cast<const V*>(s.b), max_nvec, die_local_tiles, write_through);
+      Launch(AlignedOneSegmentKernel<V, THREADS, true>, grid, dim3(THREADS), stream, e0, e1, static_cast<V*>(s.dst), static_cast<const V*>(s.a),
+             static_cast<const V*>(s.b), max_nvec, die_local_tiles, write_through);
     else
-      hipLaunchKernelGGL((AlignedOneSegmentKernel<u32x4, THREADS, false>), grid, dim3(THREADS), 0, stream, static_cast<u32x4*>(s.dst),
-                         static_cast<const u32x4*>(s.a), static_cast<const u32x4*>(nullptr), max_nvec, die_local_tiles, write_through);
+      Launch(AlignedOneSegmentKernel<u32x4, THREADS, false>, grid, dim3(THREADS), stream, e0, e1, static_cast<u32x4*>(s.dst),
+             static_cast<const u32x4*>(s.a), static_cast<const u32x4*>(nullptr), max_nvec, die_local_tiles, write_through);
   } else {
     const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, die_local_tiles, write_through);
-    if (add) hipLaunchKernelGGL((AlignedSegmentKernel<V, PER_VEC, THREADS, true>), grid, dim3(THREADS), 0, stream, args);
-    else hipLaunchKernelGGL((AlignedSegmentKernel<u32x4, PER_VEC, THREADS, false>), grid, dim3(THREADS), 0, stream, args);
+    if (add) Launch(AlignedSegmentKernel<V, PER_VEC, THREADS, true>, grid, dim3(THREADS), stream, e0, e1, args);
+    else Launch(AlignedSegmentKernel<u32x4, PER_VEC, THREADS, false>, grid, dim3(THREADS), stream, e0, e1, args);
   }
   return hipGetLastError();
 }
 
 template <typename V, int PER_VEC>
-hipError_t LaunchAligned(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream) {
-  return shape.threads == 256 ? LaunchAlignedOne<V, PER_VEC, 256>(batch, max_nvec, add, shape, stream)
-                              : LaunchAlignedOne<V, PER_VEC, 128>(batch, max_nvec, add, shape, stream);
+hipError_t LaunchAligned(const SegmentBatch& batch, uint64_t max_nvec, bool add, const LaunchShape& shape, hipStream_t stream, hipEvent_t e0,
+                         hipEvent_t e1) {
+  return shape.threads == 256 ? LaunchAlignedOne<V, PER_VEC, 256>(batch, max_nvec, add, shape, stream, e0, e1)
+                              : LaunchAlignedOne<V, PER_VEC, 128>(batch, max_nvec, add, shape, stream, e0, e1);
 }
 
 template <typename T, typename V, int THREADS, bool ADD>
-hipError_t LaunchPeeledOne(const SegmentBatch& batch, uint64_t max_n, const LaunchShape& shape, hipStream_t stream) {
+hipError_t LaunchPeeledOne(const SegmentBatch& batch, uint64_t max_n, const LaunchShape& shape, hipStream_t stream, hipEvent_t e0, hipEvent_t e1) {
   uint64_t blocks = (max_n / (16 / sizeof(T)) + THREADS - 1) / THREADS;
   if (blocks == 0) blocks = 1;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
@@ -199,21 +218,23 @@ hipError_t LaunchPeeledOne(const SegmentBatch& batch, uint64_t max_n, const Laun
   const uint32_t write_through = shape.write_through ? 1u : 0u;
   if (batch.count == 1) {
     const Segment& s = batch.seg[0];
-    hipLaunchKernelGGL((OneSegmentKernel<T, V, THREADS, ADD>), grid, dim3(THREADS), 0, stream, static_cast<T*>(s.dst), static_cast<const T*>(s.a),
-                       static_cast<const T*>(s.b), s.n, die_local_tiles, write_through);
+    Launch(OneSegmentKernel<T, V, THREADS, ADD>, grid, dim3(THREADS), stream, e0, e1, static_cast<T*>(s.dst), static_cast<const T*>(s.a),
+           static_cast<const T*>(s.b), static_cast<uint64_t>(s.n), die_local_tiles, write_through);
   } else {
     const KernelSegments<kMaxSegments> args = MakeKernelSegments<kMaxSegments>(batch, die_local_tiles, write_through);
-    hipLaunchKernelGGL((SegmentKernel<T, V, THREADS, ADD>), grid, dim3(THREADS), 0, stream, args);
+    Launch(SegmentKernel<T, V, THREADS, ADD>, grid, dim3(THREADS), stream, e0, e1, args);
   }
   return hipGetLastError();
 }
 
 // A copy moves bits: the element types of one width share a copy kernel (CopyT, CopyV).
 template <typename T, typename V, typename CopyT, typename CopyV>
-hipError_t LaunchPeeled(const SegmentBatch& batch, uint64_t max_n, bool add, const LaunchShape& shape, hipStream_t stream) {
+hipError_t LaunchPeeled(const SegmentBatch& batch, uint64_t max_n, bool add, const LaunchShape& shape, hipStream_t stream, hipEvent_t e0, hipEvent_t e1) {
   if (shape.threads == 256)
-    return add ? LaunchPeeledOne<T, V, 256, true>(batch, max_n, shape, stream) : LaunchPeeledOne<CopyT, CopyV, 256, false>(batch, max_n, shape, stream);
-  return add ? LaunchPeeledOne<T, V, 128, true>(batch, max_n, shape, stream) : LaunchPeeledOne<CopyT, CopyV, 128, false>(batch, max_n, shape, stream);
+    return add ? LaunchPeeledOne<T, V, 256, true>(batch, max_n, shape, stream, e0, e1)
+               : LaunchPeeledOne<CopyT, CopyV, 256, false>(batch, max_n, shape, stream, e0, e1);
+  return add ? LaunchPeeledOne<T, V, 128, true>(batch, max_n, shape, stream, e0, e1)
+             : LaunchPeeledOne<CopyT, CopyV, 128, false>(batch, max_n, shape, stream, e0, e1);
 }
 
 }  // namespace
@@ -275,7 +296,7 @@ hipError_t DescribeLaunch(const SegmentBatch& given, int dtype, LaunchShape* sha
   return Prepare(given, dtype, &batch, shape, &max_n);
 }
 
-hipError_t LaunchSegments(const SegmentBatch& given, int dtype, hipStream_t stream) {
+hipError_t LaunchSegments(const SegmentBatch& given, int dtype, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
   SegmentBatch batch;
   LaunchShape shape;
   uint64_t max_n = 0;
@@ -287,19 +308,19 @@ hipError_t LaunchSegments(const SegmentBatch& given, int dtype, hipStream_t stre
   if (shape.aligned) {
     const uint64_t max_nvec = max_n / per_vec;
     switch (dtype) {
-      case kF32: return LaunchAligned<f32x4, 4>(batch, max_nvec, add, shape, stream);
-      case kI32: return LaunchAligned<u32x4, 4>(batch, max_nvec, add, shape, stream);
-      case kF64: return LaunchAligned<f64x2, 2>(batch, max_nvec, add, shape, stream);
-      case kI64: return LaunchAligned<u64x2, 2>(batch, max_nvec, add, shape, stream);
+      case kF32: return LaunchAligned<f32x4, 4>(batch, max_nvec, add, shape, stream, start, stop);
+      case kI32: return LaunchAligned<u32x4, 4>(batch, max_nvec, add, shape, stream, start, stop);
+      case kF64: return LaunchAligned<f64x2, 2>(batch, max_nvec, add, shape, stream, start, stop);
+      case kI64: return LaunchAligned<u64x2, 2>(batch, max_nvec, add, shape, stream, start, stop);
       default: return hipErrorInvalidValue;
     }
   }
 
   switch (dtype) {
-    case kF32: return LaunchPeeled<float, f32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream);
-    case kI32: return LaunchPeeled<uint32_t, u32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream);
-    case kF64: return LaunchPeeled<double, f64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream);
-    case kI64: return LaunchPeeled<uint64_t, u64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream);
+    case kF32: return LaunchPeeled<float, f32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream, start, stop);
+    case kI32: return LaunchPeeled<uint32_t, u32x4, uint32_t, u32x4>(batch, max_n, add, shape, stream, start, stop);
+    case kF64: return LaunchPeeled<double, f64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream, start, stop);
+    case kI64: return LaunchPeeled<uint64_t, u64x2, uint64_t, u64x2>(batch, max_n, add, shape, stream, start, stop);
     default: return hipErrorInvalidValue;
   }
 }

@@ -13,8 +13,9 @@
 // copy.  The work is pure HBM streaming: 12 bytes per fp32 element for the
 // two-source add, 8 for a copy; there is nothing for MFMA or LDS to do.  Each
 // lane moves one 16-byte vector per operand (global_load_dwordx4 /
-// global_store_dwordx4), loads with the non-temporal hint, stores written
-// through to the memory-side cache.
+// global_store_dwordx4), loads with the non-temporal hint, stores with the
+// agent-scope bit (sc1) while a launch writes little enough for the cache in
+// front of HBM to take it, non-temporal beyond.
 //
 // Two kernels share that contract.  AlignedSegmentKernel takes the launches in which every pointer
 // is on a 16-byte boundary (dst on a 128-byte one) and every length a whole number of vectors (in practice all of the
@@ -49,14 +50,16 @@ struct LaunchShape {
   bool aligned;    // AlignedSegmentKernel (true) or SegmentKernel (false)
   int threads;     // workgroup size: 256, or 128 for large segments
   bool die_local;  // tiles ordered so that each die gets runs of 8 consecutive tiles
-  bool write_through;  // vector stores written through the memory-side cache instead of past it
+  bool write_through;  // vector stores carry sc1 (agent scope: past the die's L2, into the memory-side cache) instead of the non-temporal hint
   int segments;    // non-empty segments
 };
 
 // Enqueue one launch covering batch.seg[0..count).  Empty segments are legal; all segments of a
 // launch must be of one kind (every b set: add, every b null: copy).
-// Returns the HIP error of the launch.
-hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, hipStream_t stream);
+// Returns the HIP error of the launch.  `start` and `stop`, when given (events created with timing), receive
+// the kernel's own begin and end timestamps; the time between them is the kernel's duration.  A launch
+// with nothing to do leaves them untouched.
+hipError_t LaunchSegments(const SegmentBatch& batch, int dtype, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 // How LaunchSegments would issue this batch, without launching anything.
 hipError_t DescribeLaunch(const SegmentBatch& batch, int dtype, LaunchShape* shape);
 

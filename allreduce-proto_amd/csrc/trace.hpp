@@ -17,8 +17,9 @@
 //   other               Begin / Finish of a collective; in a graph replay, the call that launches
 //                       the graph and the wait for its completion flag
 //
-// Beyond the reference: three more lines in the same format hold DEVICE durations, measured with
-// HIP events on the streams the work ran on:
+// Beyond the reference: when device work was traced, three more lines in the same format hold DEVICE
+// durations, measured with HIP events on the streams the work ran on (without any, the file has the
+// reference's seven lines and nothing else):
 //   device-redu-kernel  each reduction launch (eager issue only)
 //   device-copy-kernel  each landing copy and each gather (eager issue only)
 //   device-graph        each replay of a recorded call, first kernel to last
@@ -90,8 +91,13 @@ class Trace {
       for (size_t i = 0; i + 1 < v.size(); i += 2) out << Millis(base_, v[i]) << "," << Millis(v[i], v[i + 1]) << ",";
       out << std::endl;
     }
+    // The reference's file ends here.  The device lines follow only when there is something to put
+    // in them, so a consumer that expects the seven lines finds exactly those unless device work
+    // was traced.
+    bool any_device = false;
+    for (int c = 0; c < kDeviceCategories; c++) any_device = any_device || !device_[c].empty();
     static const char* device_names[kDeviceCategories] = {"device-redu-kernel", "device-copy-kernel", "device-graph"};
-    for (int c = 0; c < kDeviceCategories; c++) {
+    for (int c = 0; any_device && c < kDeviceCategories; c++) {
       out << device_names[c] << ",";
       for (double x : device_[c]) out << x << ",";
       out << std::endl;

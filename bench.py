@@ -1,12 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X allreduce hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5] [--no-others] [--all-configs]
     python bench.py --only-roofline [--config N]     the kernel leg alone (what the counter profiles run)
     python bench.py --whole-buffer                    adds roofline.whole_buffer_launch to the line
     python bench.py --sweep [--config N]              every kernel variant of the measurement library at the launch shape
     python bench.py --ceiling [--config N]            the best variant, the shipped kernel on a large launch, hipMemcpyAsync
-    python bench.py --overlap [--config N]            other ways to issue a schedule of dependent launches, and to wait for it
     python bench.py --call-breakdown [--config N]     where the time of one blocking call goes, from the library's own trace
 
 One "step" is one rank's complete allreduce schedule on the GPU -- one GPU's share of the
@@ -27,9 +26,17 @@ Two more legs, both on rank 0 of a one-GPU run:
                 gcc -O2, one thread per emulated rank) on the same workload, timed on the host.
 The oracle is used only as that baseline and as the checker of the final result.
 
---sweep, --ceiling and --overlap use libibcomm_hip_bench.so (allreduce-proto_amd/csrc/bench_variants.hip):
-alternative forms of the kernel and probes of other issue schemes, built for measuring only; the default
-run loads it for `roofline.ceiling` (the best of those forms at the launch shape, next to the shipped kernel).
+The default run also carries, under `extra`:
+  other_configs   configurations 4 and 3 (5 with --all-configs) measured the same way after the headline one: rank
+                  and whole-world time per step, the kernel-landing variant, and the roofline leg of their dominant launch
+  reference_api   the reference's own entry point and protocol: the example program built against the drop-in header,
+                  one thread per rank in blocking AllreduceRingCuda calls, 3 warm-ups then timed calls, configurations 2 and 4
+and under `roofline`, `in_schedule_*`: the kernels' own durations inside the rank's schedule, taken from the
+library's trace of eagerly issued calls (each launch leaves its own begin and end timestamps there).
+
+--sweep and --ceiling use libibcomm_hip_bench.so (allreduce-proto_amd/csrc/bench_variants.hip): alternative
+forms of the kernel, built for measuring only; the default run loads it for `roofline.ceiling` (the best of
+those forms at the launch shape, next to the shipped kernel).
 """
 import argparse
 import ctypes as C
@@ -47,7 +54,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # each calibrated against a device copy of known size; the summaries with the commands are under
 # profiles/.  Shapes that have not been measured report null.
 MEASURED_TRAFFIC_BYTES = {
-    # (launch shape, workgroup size, die-local tile order, written-through stores) of the aligned kernel -> bytes;
+    # (launch shape, workgroup size, die-local tile order, sc1 stores) of the aligned kernel -> bytes;
     # all four from profiles/aligned_add_kernel_traffic_four_configs.md
     ("1 segments x 8388608 fp32", 128, 1, 1): 100676300,     # config 2
     ("2 segments x 25165824 fp32", 128, 1, 0): 603980781,    # config 3
@@ -190,7 +197,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches, sta
         "traffic": MEASURED_TRAFFIC_BYTES.get((shape, threads.value, die_local.value, through.value)) if aligned.value else None,
         "kernel": "ibcomm_hip::%s<float4, %d threads, add>, %s tile order, non-temporal loads, %s stores" % (
             ("Aligned" if aligned.value else "") + ("OneSegmentKernel" if k == 1 else "SegmentKernel"), threads.value,
-            "die-local" if die_local.value else "plain", "written-through (sc1)" if through.value else "non-temporal"),
+            "die-local" if die_local.value else "plain", "agent-scope (sc1)" if through.value else "non-temporal"),
         "launch_shape": shape,
         "algorithmic_bytes_per_launch": int(algorithmic),
         "avg_launch_us": round(avg_s * 1e6, 2),
@@ -200,7 +207,7 @@ def roofline_leg(torch, H, send, recv, seg_elems, segs_per_launch, launches, sta
     }
 
 
-# ---- the measurement library: kernel variants and issue-mode probes --------------------------------
+# ---- the measurement library: kernel variants -------------------------------------------------------
 
 _bench_lib = None
 
@@ -212,15 +219,12 @@ def bench_lib():
         if not os.path.exists(path):
             raise RuntimeError("%s is not built; run __graft_entry__.build()" % path)
         B = C.CDLL(path)
-        vp, sz, i, dp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)
+        vp, sz, i = C.c_void_p, C.c_size_t, C.c_int
         B.ibv_last_error.restype = C.c_char_p
         B.ibv_variant_name.restype = C.c_char_p
         B.ibv_variant_name.argtypes = [i]
         B.ibv_variant_accepts.argtypes = [i, sz]
         B.ibv_variant_launch.argtypes = [i, vp, vp, vp, sz, vp]
-        B.ibv_probe_chains.argtypes = [i, vp, vp, vp, sz, sz, i, i, i, dp]
-        B.ibv_probe_flags.argtypes = [i, i, vp, vp, vp, sz, sz, i, i, dp, C.POINTER(i)]
-        B.ibv_probe_blocking_call.argtypes = [i, vp, vp, vp, sz, sz, i, i, dp]
         _bench_lib = B
     return _bench_lib
 
@@ -382,57 +386,6 @@ def print_variant_table(title, times, bytes_per_launch):
         print("%-100s %10.2f %10.1f %8.4f" % (name, t * 1e6, bytes_per_launch / t * 1e-9, bytes_per_launch / t * 1e-9 / HBM_PEAK_GBPS), flush=True)
 
 
-def overlap_leg(torch, send, recv, seg_elems):
-    """Other ways to issue 14 dependent steps of the launch shape (one rank's ring schedule has 14), and to wait for them."""
-    B = bench_lib()
-    n = send[0].numel()
-    region = n * 4
-    ra, rb, rd = send[0].data_ptr(), send[1].data_ptr(), recv[0].data_ptr()
-    steps = 14
-    us = C.c_double()
-    gave_up = C.c_int()
-
-    def chains(mode, k):
-        assert B.ibv_probe_chains(mode, ra, rb, rd, region, seg_elems, steps, k, 20, C.byref(us)) == 0, B.ibv_last_error()
-        return us.value
-
-    def blocking(method, iters=100):
-        assert B.ibv_probe_blocking_call(method, ra, rb, rd, region, seg_elems, steps, iters, C.byref(us)) == 0, B.ibv_last_error()
-        return us.value
-
-    base = chains(0, 1)
-    print("%d dependent steps of dst = a + b on %d fp32 each (%.1f MB of traffic per step), device pace" % (steps, seg_elems, 12e-6 * seg_elems))
-    print("%-96s %10s %10s %8s" % ("how the steps are issued", "us/sched.", "us/step", "of peak"))
-
-    def row(name, t):
-        print("%-96s %10.2f %10.2f %8.4f" % (name, t, t / steps, 12.0 * seg_elems * steps / t * 1e-3 / HBM_PEAK_GBPS), flush=True)
-
-    row("one stream, in-order launches (what the engine issues; a recorded graph is one such chain)", base)
-    row("one stream, launches without the implicit barrier (hipExtAnyOrderLaunch; ignores the dependency)", chains(1, 1))
-    row("one stream, every 2nd launch without the implicit barrier (steps two apart still ordered)", chains(4, 2))
-    for k in (1, 2, 4, 8):
-        row("HIP graph of kernel nodes, %d parallel chain(s), each 1/%d of every step" % (k, k), chains(2, k))
-    for k in (2, 4):
-        row("%d streams issued eagerly, each 1/%d of every step" % (k, k), chains(3, k))
-    for flags, any_order, name in ((0, 0, "kernel with the counters' operands but neither signal nor wait"),
-                                   (1, 0, "every wave signals its chunk's ready counter (4 chunks per step)"),
-                                   (3, 0, "... and every workgroup waits for the previous step's counter of its chunk"),
-                                   (3, 1, "... the same, launched without the implicit barrier")):
-        assert B.ibv_probe_flags(flags, any_order, ra, rb, rd, region, seg_elems, steps, 10, C.byref(us), C.byref(gave_up)) == 0, B.ibv_last_error()
-        row(name + (" [some waits gave up]" if gave_up.value else ""), us.value)
-    print()
-    null_pace = blocking(6)
-    print("a kernel boundary on one in-order stream: %d empty kernels back to back take %.2f us, %.2f us each" % (steps, null_pace, null_pace / steps))
-    print("one blocking call = issue the %d steps and return when they are done; host wall time per call, minus the device pace above (%.2f us):" % (steps, base))
-    for method, name in ((0, "launches + hipStreamSynchronize"), (1, "launches + spin on hipStreamQuery"),
-                         (2, "launches + a one-thread kernel writing a flag in pinned host memory, host spins on the flag"),
-                         (3, "graph replay + hipStreamSynchronize"), (4, "graph replay, then the flag kernel launched behind it, host spins on the flag"),
-                         (9, "graph whose last node stores the device clock to pinned host memory, host spins (what the library does)"),
-                         (7, "graph replay + hipStreamWriteValue64 of the flag (no kernel), host spins on the flag")):
-        t = blocking(method)
-        print("    %-100s %8.2f us per call, %6.2f over device pace" % (name, t, t - base), flush=True)
-
-
 def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
     """Where one blocking call of the rank's schedule spends its time, from the library's trace: per-launch device
     durations when the call is issued eagerly, and for graph replays the host spans "graph launched" and "waiting for
@@ -456,7 +409,8 @@ def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
         t = wall(calls)
         w.dump_trace()
         w.set_trace(False)
-        lines = {ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in open("%s_%d.dat" % (base, rank)).read().splitlines()}
+        lines = {name: [] for name in ("device-redu-kernel", "device-copy-kernel", "device-graph")}  # written only when device work was timed
+        lines.update({ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in open("%s_%d.dat" % (base, rank)).read().splitlines()})
         return t, lines
 
     for _ in range(5):
@@ -489,91 +443,100 @@ def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
     w.set_graph_mode(1)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
-    ap.add_argument("--landing", choices=["memcpy", "kernel", "direct", "staged"], default=None)
-    ap.add_argument("--fuse", type=int, default=None)
-    ap.add_argument("--no-graph", action="store_true", help="issue every step eagerly instead of replaying a HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
-    ap.add_argument("--only-roofline", action="store_true",
-                    help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
-    ap.add_argument("--leg-shape", default=None, metavar="SEGMENTS,ELEMENTS,STAGING_ELEMENTS",
-                    help="with --only-roofline: time exactly this launch shape (as printed by a plain --only-roofline run as "
-                         "`leg_shape`) without running the collective first, so that a profile of the command holds the leg's launches only")
-    ap.add_argument("--whole-buffer", action="store_true",
-                    help="also time the reduction kernel over one whole per-rank buffer in a single segment "
-                         "(roofline.whole_buffer_launch): what it sustains once a launch is large")
-    ap.add_argument("--sweep", action="store_true",
-                    help="time every kernel variant of the measurement library, adds and copies, at the workload's launch shape")
-    ap.add_argument("--ceiling", action="store_true",
-                    help="the best variant at the launch shape, the shipped kernel on a whole-buffer launch, and hipMemcpyAsync")
-    ap.add_argument("--call-breakdown", action="store_true",
-                    help="run the rank's schedule with the library's trace on, eagerly and as graph replays, and print host spans "
-                         "and device durations per call")
-    ap.add_argument("--overlap", action="store_true",
-                    help="other ways of issuing the schedule's dependent launches (graph chains, streams, no-barrier launches, "
-                         "ready counters) and of waiting for them")
-    args = ap.parse_args()
+def same_bits(torch, got, want, what, chunk_elems):
+    """Bit-exact comparison of two device tensors; a mismatch is described on stderr (how many elements, where)."""
+    bad = got.view(torch.int32) != want.view(torch.int32)
+    count = int(bad.sum())
+    if count == 0:
+        return True
+    where = bad.nonzero().flatten()
+    first, last = int(where[0]), int(where[-1])
+    print("PARITY MISMATCH in %s: %d of %d elements differ, first %d (chunk %d), last %d (chunk %d); got %r want %r" % (
+        what, count, got.numel(), first, first // chunk_elems, last, last // chunk_elems, float(got[first]), float(want[first])),
+        file=sys.stderr, flush=True)
+    return False
 
-    if args.gpus != 1:
-        print("bench.py measures one GPU only: every emulated rank lives on the same MI355X and nothing in this build "
-              "uses a second device; run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py is a single-process, single-GPU benchmark; do not launch it under torchrun", file=sys.stderr)
-        sys.exit(2)
 
-    import torch
-    import hip_lib as H
-    import oracle_lib as O
+def timed(torch, H, call, steps, warm):
+    for _ in range(warm):
+        assert call() == 0, H.last_error()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rc = call()
+        assert rc == 0, H.last_error()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
 
-    algo_name, world, n, chunk, kind = CONFIGS[args.config]
+
+def device_bytes(s):
+    return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
+
+
+def in_schedule_leg(torch, H, w, rank, algo, send_ptr, out_ptr, n, calls=10):
+    """The kernels' own durations inside the rank's schedule: the schedule issued eagerly with the library's trace on,
+    where every launch leaves its begin and end timestamps (the dispatch's own, as a profiler reports them) in the
+    trace's device lines.  -> per-position means over `calls` calls, reductions and gathers in the order launched."""
+    import tempfile
+    base = os.path.join(tempfile.mkdtemp(), "trace")
+    saved = os.environ.get("IBCOMM_TRACE_FILE")
+    os.environ["IBCOMM_TRACE_FILE"] = base
+    w.set_graph_mode(0)
+    try:
+        for _ in range(2):
+            assert w.replay(rank, algo, H.F32, send_ptr, out_ptr, n) == 0, H.last_error()
+        w.set_trace(True)
+        for _ in range(calls):
+            assert w.replay(rank, algo, H.F32, send_ptr, out_ptr, n) == 0, H.last_error()
+        w.dump_trace()
+        w.set_trace(False)
+    finally:
+        w.set_graph_mode(1)
+        if saved is None:
+            os.environ.pop("IBCOMM_TRACE_FILE", None)
+        else:
+            os.environ["IBCOMM_TRACE_FILE"] = saved
+    lines = {name: [] for name in ("device-redu-kernel", "device-copy-kernel")}
+    lines.update({ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in open("%s_%d.dat" % (base, rank)).read().splitlines()})
+
+    def per_position(durations_ms):
+        k = len(durations_ms) // calls
+        if k == 0:
+            return []
+        return [round(sum(durations_ms[c * k + i] for c in range(calls)) / calls * 1e3, 2) for i in range(k)]
+
+    return per_position(lines["device-redu-kernel"][1::2]), per_position(lines["device-copy-kernel"][1::2])
+
+
+def measure_config(torch, H, O, cfg, args, steps, warm, full):
+    """One configuration: the whole world once (recorded, checked), rank 0's schedule replayed and timed, the whole
+    world timed, the kernel-landing variant, the roofline legs.  `full` adds the legs only the headline configuration
+    carries (hipMemcpyAsync landing, the ceiling).  -> dict of everything measured."""
+    algo_name, world, n, chunk, kind = CONFIGS[cfg]
     algo = H.RING if algo_name == "ring" else H.RABENSEIFNER
-    torch.cuda.set_device(0)
     os.environ["IBCOMM_CHUNKSIZE"] = str(chunk)
-    if args.config == 4:
+    if cfg == 4:
         os.environ.setdefault("IBCOMM_NUM_CUDA_STREAM", "64")
-
+    landing_name = args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")
+    rank = 0
     send = make_inputs(torch, world, n, kind, 1234)
     recv = [torch.empty_like(t) for t in send]
+    # The library's streams do not synchronise with torch's: the inputs must be complete (and torch's
+    # allocator done recycling the generators' temporaries under these very addresses) before it runs.
+    torch.cuda.synchronize()
     sp = [t.data_ptr() for t in send]
     rp = [t.data_ptr() for t in recv]
+    res = {"cfg": cfg, "algo_name": algo_name, "world": world, "n": n, "chunk": chunk, "rank": rank, "landing": landing_name}
 
-    def timed(call, steps, warm):
-        for _ in range(warm):
-            assert call() == 0, H.last_error()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            rc = call()
-            assert rc == 0, H.last_error()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / steps
-
-    if args.only_roofline and args.leg_shape:
-        k, elems, staging_elems = (int(x) for x in args.leg_shape.split(","))
-        staging = torch.empty(max(staging_elems, k * elems), device="cuda")
-        for _ in range(3):  # the copies of known size that calibrate hardware counters (see below)
-            recv[0].copy_(send[0])
-        torch.cuda.synchronize()
-        print(json.dumps({"only_roofline": True, "config": args.config, "leg_shape": args.leg_shape,
-                          "roofline": roofline_leg(torch, H, send, recv, elems, k, 200, staging)}))
-        return
-
-    rank = 0
-    with H.World(world) as w:
+    w = H.World(world)
+    keep_open = False
+    try:
         if args.landing:
             w.set_landing({"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT, "staged": H.LAND_STAGED}[args.landing])
         if args.fuse:
             w.set_max_fuse(args.fuse)
         if args.no_graph:
             w.set_graph_mode(0)
-        warm = max(args.warmup, 0 if args.no_graph else 2)  # the call shape is recorded on its second use
 
         # 1. the whole world once, eagerly, recording what `rank` receives; its counters give the per-step work
         w.reset_stats()
@@ -581,9 +544,13 @@ def main():
         torch.cuda.synchronize()
         st = [w.stats(r) for r in range(world)]
         parity = check_result(torch, O, H, algo, send, recv, chunk)
+        if not parity:
+            print("PARITY MISMATCH in config %d: the whole world's result differs from the oracle / from torch's adds in the reference's order" % cfg,
+                  file=sys.stderr, flush=True)
 
         # 2. THE TIMED STEP: `rank`'s complete schedule on its own, peers replaced by the recording
         out = torch.empty_like(send[rank])
+        torch.cuda.synchronize()
         w.reset_stats()
         assert w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n) == 0, H.last_error()
         st_rank = w.stats(rank)
@@ -604,11 +571,226 @@ def main():
         if st_rank["largest_reduce_launches"] < 2:
             staging_elems = max(staging_elems, written_per_call)
         staging = torch.empty(max(staging_elems, seg_elems * leg_segments), device="cuda")
+        res.update(send=send, recv=recv, staging=staging, seg_elems=seg_elems, leg_segments=leg_segments, st=st, st_rank=st_rank, w=w,
+                   algo=algo, sp=sp, rp=rp, out=out)
+        if args.call_breakdown or args.sweep or args.ceiling or args.only_roofline:
+            keep_open = True
+            return res  # the caller runs its leg inside this world, then closes it
 
-        if args.call_breakdown:
-            call_breakdown(torch, H, w, rank, algo, sp[rank], out.data_ptr(), n)
-            return
-        if args.sweep or args.ceiling or args.overlap:
+        # the C entry point with its arguments converted once, as any caller in a loop would hold them
+        replay_fn = H.lib().ibcomm_hip_replay_allreduce
+        replay_args = (w.comms[rank], C.c_int(algo), C.c_int(H.F32), C.c_void_p(sp[rank]), C.c_void_p(out.data_ptr()), C.c_size_t(n))
+        res["sec_per_step"] = timed(torch, H, lambda: replay_fn(*replay_args), steps, warm)
+        parity = same_bits(torch, out, recv[rank], "config %d, rank schedule replayed" % cfg, chunk // 4) and parity
+
+        # 3. for reference: all ranks' schedules executed on the one GPU per step
+        res["world_sec"] = timed(torch, H, lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), steps, warm)
+        res["graph_counters"] = w.graph_counters()
+
+        # 4. the kernels' own durations inside the schedule (eager issue, traced)
+        if not args.no_graph:
+            res["in_schedule_reduce_us"], res["in_schedule_copy_us"] = in_schedule_leg(torch, H, w, rank, algo, sp[rank], out.data_ptr(), n)
+            parity = same_bits(torch, out, recv[rank], "config %d, rank schedule issued eagerly with the trace on" % cfg, chunk // 4) and parity
+
+        # 5. for reference: the same single-rank schedule when every message is first copied into a pool
+        #    slot of the receiver by a copy kernel ("kernel" landing), unless that is the mode already measured
+        res["copied"] = None
+        if landing_name != "kernel":
+            w.set_landing(H.LAND_KERNEL)
+            out.fill_(0)
+            torch.cuda.synchronize()
+            copied_sec = timed(torch, H, lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), steps, warm)
+            copied_ok = same_bits(torch, out, recv[rank], "config %d, kernel landing" % cfg, chunk // 4)
+            parity = parity and copied_ok
+            res["copied"] = {"ms_per_step": round(copied_sec * 1e3, 4), "algbw_GBps": round(n * 4 / copied_sec * 1e-9, 2),
+                             "parity_bit_exact": copied_ok}
+
+        # 6. and the most literal form: every message lands in a pool slot through hipMemcpyAsync
+        #    (always issued eagerly), unless that is the mode already measured
+        res["memcpy_landing"] = None
+        if full and landing_name != "memcpy":
+            w.set_landing(H.LAND_MEMCPY)
+            out.fill_(0)
+            torch.cuda.synchronize()
+            w.reset_stats()
+            m_sec = timed(torch, H, lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), min(steps, 10), 2)
+            calls = w.stats(rank)["calls"]
+            copies = (w.stats(rank)["landing_copies"] + w.stats(rank)["gather_copies"]) // max(1, calls)
+            m_ok = same_bits(torch, out, recv[rank], "config %d, hipMemcpyAsync landing" % cfg, chunk // 4)
+            parity = parity and m_ok
+            res["memcpy_landing"] = {"ms_per_step": round(m_sec * 1e3, 4), "algbw_GBps": round(n * 4 / m_sec * 1e-9, 2),
+                                     "hipMemcpyAsync_calls_per_step": copies, "parity_bit_exact": m_ok}
+    finally:
+        if not keep_open:
+            w.close()
+            res["w"] = None
+    res["parity"] = parity
+
+    # 7. the dominant kernel at its in-schedule launch shape
+    if not args.no_roofline:
+        leg = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)
+        # the same launches with the result walking through all ranks' recvbufs instead (2 GiB and more): what
+        # the one reduction per schedule whose result stays in recvbuf sees
+        far = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
+        leg["result_walking_through_all_recvbufs"] = {k: far[k] for k in ("avg_launch_us", "achieved", "frac")}
+        if "in_schedule_reduce_us" in res and res["in_schedule_reduce_us"]:
+            # mean over the rank's reduction launches of the dominant shape, as they ran inside the schedule
+            dominant = [u for u in res["in_schedule_reduce_us"]]
+            mean_us = sum(dominant) / len(dominant)
+            alg = 12.0 * st_rank["reduce_elements"] / len(dominant)
+            leg["in_schedule_what"] = ("each launch's own begin-to-end time inside rank 0's schedule, the schedule issued eagerly (pool streams in turn, "
+                                       "event-ordered) with the library's trace on, mean over 10 calls per position; a graph replay runs the same launches as one chain")
+            leg["in_schedule_reduce_launches_us"] = res["in_schedule_reduce_us"]
+            leg["in_schedule_mean_us"] = round(mean_us, 2)
+            leg["in_schedule_frac"] = round(alg / (mean_us * 1e-6) * 1e-9 / HBM_PEAK_GBPS, 4)
+            leg["in_schedule_gather_launches_us"] = res["in_schedule_copy_us"]
+        leg["target_0p80_met"] = bool(leg["frac"] >= 0.80)
+        if full:
+            leg["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], staging=staging)
+            if args.whole_buffer:
+                # the same kernel over one whole per-rank buffer: what it sustains once the launch is large.
+                # Not part of the default run, so that a profile of the default run holds the dominant
+                # shape only under this kernel's name.
+                whole = roofline_leg(torch, H, send, recv, n, 1, 40)
+                leg["whole_buffer_launch"] = {k: whole[k] for k in (
+                    "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
+        res["roofline"] = leg
+    for k in ("send", "recv", "staging", "out", "sp", "rp"):
+        res.pop(k, None)
+    del send, recv, staging, out
+    torch.cuda.empty_cache()
+    return res
+
+
+def summary_of(res):
+    """The figures of one configuration that the measured table is made of."""
+    n, world = res["n"], res["world"]
+    rank_bytes = device_bytes(res["st_rank"])
+    world_bytes = sum(device_bytes(s) for s in res["st"])
+    out = {
+        "workload": "%s allreduce, %d emulated ranks, %d fp32 per rank, IBCOMM_CHUNKSIZE=%d" % (res["algo_name"], world, n, res["chunk"]),
+        "rank_ms_per_step": round(res["sec_per_step"] * 1e3, 4),
+        "rank_algbw_GBps": round(n * 4 / res["sec_per_step"] * 1e-9, 2),
+        "rank_device_GBps": round(rank_bytes / res["sec_per_step"] * 1e-9, 1),
+        "rank_frac_of_hbm_peak": round(rank_bytes / res["sec_per_step"] * 1e-9 / HBM_PEAK_GBPS, 4),
+        "world_all_ranks_on_one_gpu_ms_per_step": round(res["world_sec"] * 1e3, 4),
+        "world_all_ranks_on_one_gpu_algbw_GBps": round(n * 4 / res["world_sec"] * 1e-9, 2),
+        "rank_with_copy_kernel_landing": res["copied"],
+        "parity_bit_exact": res["parity"],
+    }
+    if "roofline" in res:
+        leg = res["roofline"]
+        out["roofline"] = {k: leg[k] for k in ("launch_shape", "kernel", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "traffic",
+                                               "result_walking_through_all_recvbufs", "target_0p80_met") if k in leg}
+        for k in ("in_schedule_what", "in_schedule_mean_us", "in_schedule_frac", "in_schedule_reduce_launches_us", "in_schedule_gather_launches_us"):
+            if k in leg:
+                out["roofline"][k] = leg[k]
+    return out
+
+
+def reference_api_leg(cfg, timed_runs=10):
+    """The reference's own entry point and timing protocol: one IBVerbsCommunicator per rank, one host thread per rank,
+    every rank in a blocking AllreduceRingCuda / AllreduceRabenseifnerCuda call; 3 warm-ups, then timed runs
+    (examples/allreduce.cpp:28-29, 107-118, which times one).  Runs the example program built against the drop-in
+    header in a process of its own."""
+    import subprocess
+    algo_name, world, n, chunk, _ = CONFIGS[cfg]
+    exe = os.path.join(ROOT, "allreduce-proto_amd", "allreduce_example")
+    if not os.path.exists(exe):
+        return {"error": "%s is not built" % exe}
+    env = dict(os.environ, IBCOMM_CHUNKSIZE=str(chunk))
+    if cfg == 4:
+        env.setdefault("IBCOMM_NUM_CUDA_STREAM", "64")
+    p = subprocess.run([exe, str(world), algo_name, str(n), str(timed_runs)], env=env, capture_output=True, text=True, timeout=600)
+    first, runs = None, []
+    for ln in p.stdout.splitlines():
+        if ln.startswith("elapsed time :"):
+            first = float(ln.split(":")[1].split()[0])
+        if ln.startswith("elapsed times of"):
+            runs = [float(x) for x in ln.split(":")[1].split()]
+    if p.returncode != 0 or first is None:
+        return {"error": "exit status %d: %s" % (p.returncode, (p.stdout + p.stderr)[-300:])}
+    runs = runs or [first]
+    return {
+        "workload": "%s, %d rank threads x %d fp32, IBCOMM_CHUNKSIZE=%d, integer-valued inputs as in the reference's example" % (algo_name, world, n, chunk),
+        "entry_point": "IBVerbsCommunicator::Allreduce%sCuda<float>, one blocking call per rank thread" % ("Ring" if algo_name == "ring" else "Rabenseifner"),
+        "protocol": "3 warm-ups, then %d timed calls; rank 0's wall clock around its own call" % len(runs),
+        "ms_per_allreduce_first_timed_call": round(first * 1e3, 4),
+        "ms_per_allreduce_median": round(sorted(runs)[len(runs) // 2] * 1e3, 4),
+        "ms_per_allreduce_max": round(max(runs) * 1e3, 4),
+        "algbw_GBps_median": round(n * 4 / sorted(runs)[len(runs) // 2] * 1e-9, 2),
+        "all_ranks_report_ok": p.stdout.count(" OK") == world,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
+    ap.add_argument("--landing", choices=["memcpy", "kernel", "direct", "staged"], default=None)
+    ap.add_argument("--fuse", type=int, default=None)
+    ap.add_argument("--no-graph", action="store_true", help="issue every step eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip extra.other_configs (configurations 4 and 3 measured after the headline one) and extra.reference_api")
+    ap.add_argument("--all-configs", action="store_true", help="extra.other_configs also holds configuration 5 (32 ranks x 2 GiB)")
+    ap.add_argument("--only-roofline", action="store_true",
+                    help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
+    ap.add_argument("--leg-shape", default=None, metavar="SEGMENTS,ELEMENTS,STAGING_ELEMENTS",
+                    help="with --only-roofline: time exactly this launch shape (as printed by a plain --only-roofline run as "
+                         "`leg_shape`) without running the collective first, so that a profile of the command holds the leg's launches only")
+    ap.add_argument("--whole-buffer", action="store_true",
+                    help="also time the reduction kernel over one whole per-rank buffer in a single segment "
+                         "(roofline.whole_buffer_launch): what it sustains once a launch is large")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time every kernel variant of the measurement library, adds and copies, at the workload's launch shape")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="the best variant at the launch shape, the shipped kernel on a whole-buffer launch, and hipMemcpyAsync")
+    ap.add_argument("--call-breakdown", action="store_true",
+                    help="run the rank's schedule with the library's trace on, eagerly and as graph replays, and print host spans "
+                         "and device durations per call")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: every emulated rank lives on the same MI355X and nothing in this build "
+              "uses a second device; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py is a single-process, single-GPU benchmark; do not launch it under torchrun", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import hip_lib as H
+    import oracle_lib as O
+
+    algo_name, world, n, chunk, kind = CONFIGS[args.config]
+    torch.cuda.set_device(0)
+    warm = max(args.warmup, 0 if args.no_graph else 2)  # the call shape is recorded on its second use
+
+    if args.only_roofline and args.leg_shape:
+        os.environ["IBCOMM_CHUNKSIZE"] = str(chunk)
+        send = make_inputs(torch, world, n, kind, 1234)
+        recv = [torch.empty_like(t) for t in send]
+        k, elems, staging_elems = (int(x) for x in args.leg_shape.split(","))
+        staging = torch.empty(max(staging_elems, k * elems), device="cuda")
+        for _ in range(3):  # the copies of known size that calibrate hardware counters (see below)
+            recv[0].copy_(send[0])
+        torch.cuda.synchronize()
+        print(json.dumps({"only_roofline": True, "config": args.config, "leg_shape": args.leg_shape,
+                          "roofline": roofline_leg(torch, H, send, recv, elems, k, 200, staging)}))
+        return
+
+    res = measure_config(torch, H, O, args.config, args, args.steps, warm, full=True)
+    if args.call_breakdown or args.sweep or args.ceiling or args.only_roofline:
+        # legs that run inside the world measure_config left open
+        w, send, recv, staging = res["w"], res["send"], res["recv"], res["staging"]
+        seg_elems, leg_segments, rank = res["seg_elems"], res["leg_segments"], res["rank"]
+        try:
+            if args.call_breakdown:
+                call_breakdown(torch, H, w, rank, res["algo"], res["sp"][rank], res["out"].data_ptr(), n)
             total = seg_elems * leg_segments
             if args.sweep:
                 print_variant_table("dst = a + b, %d fp32 in one segment (12 B per element)" % total,
@@ -621,63 +803,27 @@ def main():
                 print(json.dumps({"config": args.config, "roofline": leg,
                                   "ceiling": ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], full=True,
                                                          staging=staging)}))
-            if args.overlap:
-                overlap_leg(torch, send, recv, total)
-            return
-        if args.only_roofline:
-            # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
-            # counters collected over this command can be calibrated against a known traffic
-            for _ in range(3):
-                recv[0].copy_(send[0])
-            torch.cuda.synchronize()
-            print(json.dumps({"only_roofline": True, "config": args.config,
-                              "leg_shape": "%d,%d,%d" % (leg_segments, seg_elems, staging.numel()),
-                              "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)}))
-            return
-        # the C entry point with its arguments converted once, as any caller in a loop would hold them
-        replay_fn = H.lib().ibcomm_hip_replay_allreduce
-        replay_args = (w.comms[rank], C.c_int(algo), C.c_int(H.F32), C.c_void_p(sp[rank]), C.c_void_p(out.data_ptr()), C.c_size_t(n))
-        sec_per_step = timed(lambda: replay_fn(*replay_args), args.steps, warm)
-        parity = parity and bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
-        del out
+            if args.only_roofline:
+                # a plain device copy of known size (n * 4 bytes read, n * 4 written), so that hardware
+                # counters collected over this command can be calibrated against a known traffic
+                for _ in range(3):
+                    recv[0].copy_(send[0])
+                torch.cuda.synchronize()
+                print(json.dumps({"only_roofline": True, "config": args.config,
+                                  "leg_shape": "%d,%d,%d" % (leg_segments, seg_elems, staging.numel()),
+                                  "roofline": roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)}))
+        finally:
+            w.close()
+        return
 
-        # 3. for reference: all ranks' schedules executed on the one GPU per step
-        world_sec = timed(lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), args.steps, warm)
-        graph_counters = w.graph_counters()
-
-        # 4. for reference: the same single-rank schedule when every message is first copied into a pool
-        #    slot of the receiver by a copy kernel ("kernel" landing), unless that is the mode already measured
-        copied = None
-        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")) != "kernel":
-            w.set_landing(H.LAND_KERNEL)
-            out = torch.empty_like(send[rank])
-            copied_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), args.steps, warm)
-            copied_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
-            parity = parity and copied_ok
-            copied = {"ms_per_step": round(copied_sec * 1e3, 4), "algbw_GBps": round(n * 4 / copied_sec * 1e-9, 2),
-                      "parity_bit_exact": copied_ok}
-            del out
-
-        # 5. and the most literal form: every message lands in a pool slot through its own hipMemcpyAsync
-        #    (always issued eagerly), unless that is the mode already measured
-        memcpy_landing = None
-        if (args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")) != "memcpy":
-            w.set_landing(H.LAND_MEMCPY)
-            out = torch.empty_like(send[rank])
-            m_sec = timed(lambda: w.replay(rank, algo, H.F32, sp[rank], out.data_ptr(), n), min(args.steps, 10), 2)
-            m_ok = bool(torch.equal(out.view(torch.int32), recv[rank].view(torch.int32)))
-            parity = parity and m_ok
-            memcpy_landing = {"ms_per_step": round(m_sec * 1e3, 4), "algbw_GBps": round(n * 4 / m_sec * 1e-9, 2),
-                              "parity_bit_exact": m_ok}
-            del out
-
-    def device_bytes(s):
-        return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
-
+    st, st_rank, rank = res["st"], res["st_rank"], res["rank"]
+    sec_per_step, world_sec = res["sec_per_step"], res["world_sec"]
+    parity = res["parity"]
     rank_bytes = device_bytes(st_rank)
     world_bytes = sum(device_bytes(s) for s in st)
     chunks_per_launch = round(st_rank["reduce_segments"] / max(1, st_rank["reduce_launches"]), 2)
     segs_per_launch = round(st_rank["reduce_kernel_segments"] / max(1, st_rank["reduce_launches"]), 2)
+    graph_counters = res["graph_counters"]
 
     algbw = n * 4 / sec_per_step * 1e-9
     world_algbw = n * 4 / world_sec * 1e-9
@@ -700,7 +846,7 @@ def main():
                         "other ranks' messages replayed from a recording of the full world" % (
                             args.config - 1, algo_name, world, n, n * 4 / 2**20, chunk, rank),
             "algo": algo_name, "ranks": world, "elements_per_rank": n, "chunk_bytes": chunk, "measured_rank": rank,
-            "landing": args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged"),
+            "landing": res["landing"],
             "max_fuse": args.fuse or int(os.environ.get("IBCOMM_HIP_MAX_FUSE", "64")),
         },
         "parity_bit_exact": parity,
@@ -722,34 +868,28 @@ def main():
                 "device_GBps": round(world_bytes / world_sec * 1e-9, 1),
                 "frac_of_hbm_peak": round(world_bytes / world_sec * 1e-9 / HBM_PEAK_GBPS, 4),
             },
-            "rank_with_copy_kernel_landing": copied,
-            "rank_with_hipMemcpyAsync_landing": memcpy_landing,
-            "north_star_landing_mode": "memcpy (rank_with_hipMemcpyAsync_landing is that mode's figure; `value` is the '%s' mode)" % (
-                args.landing or os.environ.get("IBCOMM_HIP_LANDING", "staged")),
+            "rank_with_copy_kernel_landing": res["copied"],
+            "rank_with_hipMemcpyAsync_landing": res["memcpy_landing"],
+            "north_star_landing_mode": "memcpy (rank_with_hipMemcpyAsync_landing is that mode's figure; `value` is the '%s' mode)" % res["landing"],
             "streams_per_rank": st[0]["streams_created"],
             "issue": "hip graph replay" if graph_counters[2] > 0 else "eager",
             "graph_calls_eager_captured_replayed": list(graph_counters),
             "pool_slots_high_water": max(s["slots_high_water"] for s in st),
         },
     }
-    if not args.no_roofline:
-        line["roofline"] = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200, staging)
-        # the same launches with the result walking through all ranks' recvbufs instead (2 GiB and more): what
-        # the one reduction per schedule whose result stays in recvbuf sees
-        far = roofline_leg(torch, H, send, recv, seg_elems, leg_segments, 200)
-        line["roofline"]["result_walking_through_all_recvbufs"] = {k: far[k] for k in ("avg_launch_us", "achieved", "frac")}
-        line["roofline"]["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, line["roofline"]["avg_launch_us"],
-                                                  staging=staging)
-        if args.whole_buffer:
-            # the same kernel over one whole per-rank buffer: what it sustains once the launch is large.
-            # Not part of the default run, so that a profile of the default run holds the dominant
-            # shape only under this kernel's name.
-            whole = roofline_leg(torch, H, send, recv, n, 1, 40)
-            line["roofline"]["whole_buffer_launch"] = {k: whole[k] for k in (
-                "launch_shape", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "launches_timed")}
-    del recv, staging
+    if "roofline" in res:
+        line["roofline"] = res["roofline"]
+    if not args.no_others:
+        # the other configurations, each to the same parity check, and the reference's own blocking per-rank entry point
+        others = {}
+        for cfg in [c for c in (4, 3) + ((5,) if args.all_configs else ()) if c != args.config]:
+            r = measure_config(torch, H, O, cfg, args, args.steps, warm, full=False)
+            others["config_%d" % cfg] = summary_of(r)
+            parity = parity and r["parity"]
+        line["extra"]["other_configs"] = others
+        line["extra"]["reference_api"] = {"config_%d" % cfg: reference_api_leg(cfg) for cfg in (2, 4)}
+        line["parity_bit_exact"] = parity
     if not args.no_cpu:
-        del send
         torch.cuda.empty_cache()
         line["cpu_baseline"] = cpu_baseline_leg(O, world, n, chunk, algo_name)
         # the like-for-like GPU figure for that baseline: all N ranks' schedules on the one GPU per step

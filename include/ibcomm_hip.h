@@ -10,7 +10,12 @@
  *
  * Conventions
  *   - Plain pointers and sizes only.  Buffers passed to the allreduce and
- *     reduce calls are DEVICE pointers on the current HIP device.
+ *     reduce calls are DEVICE pointers on the current HIP device.  The
+ *     allreduce calls work on streams of their own that do not synchronise
+ *     with the caller's (the reference creates its streams with
+ *     cudaStreamNonBlocking, ibcomm/memory_pool.h:96): whatever produces
+ *     sendbuf, and any earlier use of recvbuf's memory, must have completed
+ *     before the call, as the calls themselves complete before they return.
  *   - Every function returns 0 on success or one of the reference's exit codes
  *     (ibcomm/util.h:32-42): 1 invalid argument, 2 transport error, 3 HIP
  *     error, 4 not supported.  Where the reference prints a message and calls
@@ -174,7 +179,7 @@ int ibcomm_hip_copy_segments(int dtype, int n_segments, void* const* dst, const 
 /* How ibcomm_hip_reduce_segments would issue these segments, without launching: *aligned = 1 for the
  * kernel that takes 16-byte aligned pointers (dst: 128-byte aligned) and whole vectors (0: the general kernel), *threads the
  * workgroup size, *die_local = 1 if tiles are ordered in runs per accelerator die, *write_through = 1
- * if the stores go through the memory-side cache (0: non-temporal).  Stands for the launch geometry
+ * if the stores carry the agent-scope bit sc1 (0: the non-temporal hint).  Stands for the launch geometry
  * the reference fixes at ibcomm/allreduce_cuda_impl.h:24, 116-117. */
 int ibcomm_hip_describe_launch(int dtype, int n_segments, void* const* dst, const void* const* a, const void* const* b,
                                const size_t* len_elements, int* aligned, int* threads, int* die_local, int* write_through);

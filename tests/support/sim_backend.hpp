@@ -305,7 +305,7 @@ struct SimBackend {
     Sim::Get().AddNode(s, std::move(n));
     return 0;
   }
-  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int role = 0) {
+  static int LaunchSegments(const SegmentBatch& batch, int dtype, Stream s, int role = 0, Timer = 0, Timer = 0) {
     SimNode n;
     n.kind = 2;
     n.batch = batch;

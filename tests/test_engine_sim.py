@@ -418,10 +418,9 @@ def test_trace_file_has_the_reference_format(tmp_path):
     assert rc == 0
     lines = open(path).read().splitlines()
     names = ["received", "reduced", "issue-send", "issue-copy-kernel", "issue-redu-kernel", "issue-recv", "other"]
-    # the reference's seven lines, then this build's device-duration lines (empty: the simulated device keeps no time)
-    assert [ln.split(",")[0] for ln in lines] == names + ["device-redu-kernel", "device-copy-kernel", "device-graph"]
-    assert lines[7:] == ["device-redu-kernel,", "device-copy-kernel,", "device-graph,"]
-    lines = lines[:7]
+    # exactly the reference's seven lines: the device-duration lines are written only when device work was
+    # timed, and the simulated device keeps no time
+    assert [ln.split(",")[0] for ln in lines] == names
     q = n * 4 // 1024 // world  # chunks per group
     want_pairs = {"received": 2 * (world - 1) * q, "reduced": (world - 1) * q, "issue-send": 2 * (world - 1) * q,
                   "issue-redu-kernel": (world - 1) * q, "issue-recv": (world - 1) * q, "other": 2}

@@ -68,8 +68,12 @@ DEVICE_NAMES = ["device-redu-kernel", "device-copy-kernel", "device-graph"]
 
 def read_trace(path):
     lines = open(path).read().splitlines()
-    assert [ln.split(",")[0] for ln in lines] == TRACE_NAMES + DEVICE_NAMES  # the reference's seven lines first
-    return {ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in lines}
+    # the reference's seven lines; the three device lines follow when device work was timed, else nothing does
+    assert [ln.split(",")[0] for ln in lines] in (TRACE_NAMES, TRACE_NAMES + DEVICE_NAMES)
+    t = {name: [] for name in DEVICE_NAMES}
+    t.update({ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in lines})
+    t["lines"] = len(lines)
+    return t
 
 
 def test_trace_files(tmp_path):
@@ -93,6 +97,19 @@ def test_trace_files(tmp_path):
             assert all(0 < d < 50 for d in t[name][1::2]), t[name]        # milliseconds, positive, sane
             assert t[name][0::2] == sorted(t[name][0::2])                   # launches of one rank follow one another
         assert len(t["issue-redu-kernel"]) == len(t["device-redu-kernel"])  # one host issue span per device span
+        assert t["lines"] == 10
+
+
+def test_trace_without_device_work_has_the_reference_seven_lines(tmp_path):
+    # point-to-point traffic only: nothing is timed on the device, and the file is what DumpTrace writes
+    # in the reference (ibcomm/ibverbs_communicator.cpp:183-212), seven lines
+    base = str(tmp_path / "p2p")
+    with G.env(IBCOMM_TRACE_FILE=base):
+        with H.World(2) as w:
+            w.set_trace(True)
+            w.dump_trace()
+    for r in range(2):
+        assert read_trace("%s_%d.dat" % (base, r))["lines"] == 7
 
 
 def test_trace_of_graph_replays(tmp_path):
