@@ -48,8 +48,17 @@ struct CachedGraph {
 // value costs that call a few microseconds less than asking the runtime to synchronise the stream,
 // and a clock reading needs no state on the device: replays of one world never overlap (each call
 // waits for its own), and two readings that far apart always differ.
+//
+// What the host may conclude from the new value: every kernel of the replay has finished (this node
+// comes after them in the chain, and a kernel boundary completes the stores of the kernel before
+// it).  The store is a system-scope release behind a system-scope fence, so that nothing of this
+// node is reordered after it either; the results themselves are read by later device work or device
+// copies, which the runtime orders after this stream's work in the usual way once the caller
+// synchronises or enqueues behind it.  The runtime may retire the launch a moment after the host
+// has seen the word; an executable graph is therefore only destroyed after a stream synchronisation.
 __global__ void PublishCompletion(uint64_t* host_flag) {
-  __hip_atomic_store(host_flag, static_cast<uint64_t>(wall_clock64()), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __threadfence_system();
+  __hip_atomic_store(host_flag, static_cast<uint64_t>(wall_clock64()), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 struct ibcomm_hip_fabric {

@@ -473,29 +473,38 @@ def device_bytes(s):
     return 12 * s["reduce_elements"] + 2 * s["landing_bytes"] + 2 * s["gather_bytes"]
 
 
-def in_schedule_leg(torch, H, w, rank, algo, send_ptr, out_ptr, n, calls=10):
-    """The kernels' own durations inside the rank's schedule: the schedule issued eagerly with the library's trace on,
-    where every launch leaves its begin and end timestamps (the dispatch's own, as a profiler reports them) in the
-    trace's device lines.  -> per-position means over `calls` calls, reductions and gathers in the order launched."""
+def in_schedule_leg(torch, H, world, rank, algo, sp, rp, out_ptr, n, landing=None, fuse=None, calls=10):
+    """The kernels' own durations inside the rank's schedule.  A world of its own whose ranks issue on ONE stream each and
+    eagerly: the rank's launches then follow one another on an in-order stream exactly as the nodes of the recorded graph
+    do in a replay, and with the library's trace on every launch leaves its own begin and end timestamps (the dispatch's,
+    as a profiler reports them) in the trace's device lines.  -> per-position means over `calls` calls, reductions and
+    gathers in the order launched."""
     import tempfile
     base = os.path.join(tempfile.mkdtemp(), "trace")
-    saved = os.environ.get("IBCOMM_TRACE_FILE")
+    saved = {k: os.environ.get(k) for k in ("IBCOMM_TRACE_FILE", "IBCOMM_NUM_CUDA_STREAM")}
     os.environ["IBCOMM_TRACE_FILE"] = base
-    w.set_graph_mode(0)
+    os.environ["IBCOMM_NUM_CUDA_STREAM"] = "1"
     try:
-        for _ in range(2):
-            assert w.replay(rank, algo, H.F32, send_ptr, out_ptr, n) == 0, H.last_error()
-        w.set_trace(True)
-        for _ in range(calls):
-            assert w.replay(rank, algo, H.F32, send_ptr, out_ptr, n) == 0, H.last_error()
-        w.dump_trace()
-        w.set_trace(False)
+        with H.World(world) as w:
+            if landing is not None:
+                w.set_landing(landing)
+            if fuse:
+                w.set_max_fuse(fuse)
+            w.set_graph_mode(0)
+            assert w.record(rank, algo, H.F32, sp, rp, n) == 0, H.last_error()
+            for _ in range(2):
+                assert w.replay(rank, algo, H.F32, sp[rank], out_ptr, n) == 0, H.last_error()
+            w.set_trace(True)
+            for _ in range(calls):
+                assert w.replay(rank, algo, H.F32, sp[rank], out_ptr, n) == 0, H.last_error()
+            w.dump_trace()
+            w.set_trace(False)
     finally:
-        w.set_graph_mode(1)
-        if saved is None:
-            os.environ.pop("IBCOMM_TRACE_FILE", None)
-        else:
-            os.environ["IBCOMM_TRACE_FILE"] = saved
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
     lines = {name: [] for name in ("device-redu-kernel", "device-copy-kernel")}
     lines.update({ln.split(",")[0]: [float(x) for x in ln.split(",")[1:-1]] for ln in open("%s_%d.dat" % (base, rank)).read().splitlines()})
 
@@ -583,14 +592,38 @@ def measure_config(torch, H, O, cfg, args, steps, warm, full):
         res["sec_per_step"] = timed(torch, H, lambda: replay_fn(*replay_args), steps, warm)
         parity = same_bits(torch, out, recv[rank], "config %d, rank schedule replayed" % cfg, chunk // 4) and parity
 
+        # ... and the device's own time for one replay: HIP events before and after the graph, from the library's trace
+        if not args.no_graph:
+            import tempfile
+            base = os.path.join(tempfile.mkdtemp(), "replay")
+            saved_base = os.environ.get("IBCOMM_TRACE_FILE")
+            os.environ["IBCOMM_TRACE_FILE"] = base
+            w.set_trace(True)
+            for _ in range(20):
+                assert replay_fn(*replay_args) == 0, H.last_error()
+            w.dump_trace()
+            w.set_trace(False)
+            if saved_base is None:
+                os.environ.pop("IBCOMM_TRACE_FILE", None)
+            else:
+                os.environ["IBCOMM_TRACE_FILE"] = saved_base
+            spans = [ln for ln in open("%s_%d.dat" % (base, rank)).read().splitlines() if ln.startswith("device-graph,")]
+            durations = sorted(float(x) for x in spans[0].split(",")[1:-1][1::2]) if spans else []
+            if durations:
+                res["replay_device_us"] = round(durations[len(durations) // 2] * 1e3, 2)
+
         # 3. for reference: all ranks' schedules executed on the one GPU per step
         res["world_sec"] = timed(torch, H, lambda: w.allreduce_ptrs(algo, H.F32, sp, rp, n), steps, warm)
         res["graph_counters"] = w.graph_counters()
 
-        # 4. the kernels' own durations inside the schedule (eager issue, traced)
+        # 4. the kernels' own durations inside the schedule (a one-stream world of its own, eager issue, traced)
         if not args.no_graph:
-            res["in_schedule_reduce_us"], res["in_schedule_copy_us"] = in_schedule_leg(torch, H, w, rank, algo, sp[rank], out.data_ptr(), n)
-            parity = same_bits(torch, out, recv[rank], "config %d, rank schedule issued eagerly with the trace on" % cfg, chunk // 4) and parity
+            out.fill_(0)
+            torch.cuda.synchronize()
+            landing_code = {"memcpy": H.LAND_MEMCPY, "kernel": H.LAND_KERNEL, "direct": H.LAND_DIRECT, "staged": H.LAND_STAGED}[landing_name]
+            res["in_schedule_reduce_us"], res["in_schedule_copy_us"] = in_schedule_leg(torch, H, world, rank, algo, sp, rp, out.data_ptr(), n,
+                                                                                       landing_code, args.fuse)
+            parity = same_bits(torch, out, recv[rank], "config %d, rank schedule issued eagerly on one stream with the trace on" % cfg, chunk // 4) and parity
 
         # 5. for reference: the same single-rank schedule when every message is first copied into a pool
         #    slot of the receiver by a copy kernel ("kernel" landing), unless that is the mode already measured
@@ -638,12 +671,22 @@ def measure_config(torch, H, O, cfg, args, steps, warm, full):
             dominant = [u for u in res["in_schedule_reduce_us"]]
             mean_us = sum(dominant) / len(dominant)
             alg = 12.0 * st_rank["reduce_elements"] / len(dominant)
-            leg["in_schedule_what"] = ("each launch's own begin-to-end time inside rank 0's schedule, the schedule issued eagerly (pool streams in turn, "
-                                       "event-ordered) with the library's trace on, mean over 10 calls per position; a graph replay runs the same launches as one chain")
+            leg["in_schedule_what"] = ("each launch's own begin-to-end time (the dispatch's timestamps) with rank 0's schedule issued eagerly on one in-order "
+                                       "stream, in the order a graph replay runs the same launches, the library's trace on, mean over 10 calls per position; "
+                                       "the host issues slower than the device runs, so every launch finds the device idle: a launch on its own, without the "
+                                       "kernel boundary that a chain adds (`roofline.avg_launch_us` is back to back and contains it)")
             leg["in_schedule_reduce_launches_us"] = res["in_schedule_reduce_us"]
             leg["in_schedule_mean_us"] = round(mean_us, 2)
             leg["in_schedule_frac"] = round(alg / (mean_us * 1e-6) * 1e-9 / HBM_PEAK_GBPS, 4)
             leg["in_schedule_gather_launches_us"] = res["in_schedule_copy_us"]
+            if "replay_device_us" in res:
+                # one replay of the schedule as one chain of launches on the device, completion node included; what it
+                # takes beyond the sum of the launches' own durations is the kernel boundaries of the chain
+                own = sum(res["in_schedule_reduce_us"]) + sum(res["in_schedule_copy_us"])
+                launches = len(res["in_schedule_reduce_us"]) + len(res["in_schedule_copy_us"])
+                leg["replay_device_us_per_call"] = res["replay_device_us"]
+                leg["replay_launches_per_call"] = launches
+                leg["replay_minus_launches_own_time_us_per_launch"] = round((res["replay_device_us"] - own) / max(1, launches), 2)
         leg["target_0p80_met"] = bool(leg["frac"] >= 0.80)
         if full:
             leg["ceiling"] = ceiling_leg(torch, H, send, recv, seg_elems, leg_segments, leg["avg_launch_us"], staging=staging)
@@ -682,7 +725,8 @@ def summary_of(res):
         leg = res["roofline"]
         out["roofline"] = {k: leg[k] for k in ("launch_shape", "kernel", "algorithmic_bytes_per_launch", "avg_launch_us", "achieved", "frac", "traffic",
                                                "result_walking_through_all_recvbufs", "target_0p80_met") if k in leg}
-        for k in ("in_schedule_what", "in_schedule_mean_us", "in_schedule_frac", "in_schedule_reduce_launches_us", "in_schedule_gather_launches_us"):
+        for k in ("in_schedule_what", "in_schedule_mean_us", "in_schedule_frac", "in_schedule_reduce_launches_us", "in_schedule_gather_launches_us",
+                  "replay_device_us_per_call", "replay_launches_per_call", "replay_minus_launches_own_time_us_per_launch"):
             if k in leg:
                 out["roofline"][k] = leg[k]
     return out
