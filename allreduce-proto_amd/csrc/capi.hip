@@ -69,6 +69,11 @@ struct ibcomm_hip_fabric {
     graph_max_ops = v ? strtoull(v, nullptr, 10) : 4096;
     v = getenv("IBCOMM_HIP_RENDEZVOUS");
     meet_mode = v ? atoi(v) : 1;
+    v = getenv("IBCOMM_HIP_MERGE_RANKS");
+    merge_mode = v ? atoi(v) : 1;
+    // a merged launch stays within what the kernels store with sc1: its parts were on that side
+    v = getenv("IBCOMM_HIP_MERGE_MAX_BYTES");
+    collector.set_write_limit(v ? strtoull(v, nullptr, 10) : kWriteThroughMaxBytes);
   }
   ~ibcomm_hip_fabric() {
     DropGraphs();
@@ -90,6 +95,8 @@ struct ibcomm_hip_fabric {
   Fabric<HipBackend> fabric;
   Rendezvous meet;               // where the blocking per-rank calls of this world find each other
   int meet_mode = 1;             // 0 = every rank thread runs its own engine (IBCOMM_HIP_RENDEZVOUS=0)
+  LaunchCollector<HipBackend> collector;  // merges the ranks' launches while a world is recorded (merge.hpp)
+  int merge_mode = 1;            // 0 = a recorded world keeps one launch per rank and step (IBCOMM_HIP_MERGE_RANKS=0)
   std::mutex mu;                 // guards live_comms and the graph cache against concurrent create / destroy
   int live_comms = 0;
   int graph_mode = 1;            // 0 = always issue eagerly, 1 = capture a call shape on its second use
@@ -368,8 +375,11 @@ int WorldAllreduce(ibcomm_hip_fabric* f, std::vector<Communicator<HipBackend>*>&
   // the runtime on ROCm 7.2 (gfx950), so the per-message-memcpy landing mode is never recorded.
   const bool may_record = f->graph_mode != 0 && world_size > 1 && cs[0]->landing() != kLandMemcpy;
   const GraphKey key = MakeKey(cs, algo, dtype, len, sendbufs, recvbufs, -1);
+  // `synchronize` is false exactly while the call is being recorded: all ranks then issue on the one
+  // recording stream, which is where their launches can be merged.
   return IssueCached(f, cs, key, may_record, [&](bool synchronize) {
-    return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, synchronize);
+    LaunchCollector<HipBackend>* merge = (!synchronize && f->merge_mode != 0) ? &f->collector : nullptr;
+    return RunWorld<HipBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len, synchronize, merge);
   });
 }
 
@@ -510,6 +520,24 @@ int ibcomm_hip_fabric_graph_counters(ibcomm_hip_fabric* fabric, uint64_t* eager_
   if (eager_calls) *eager_calls = fabric->eager_calls;
   if (captures) *captures = fabric->graph_captures;
   if (replays) *replays = fabric->graph_replays;
+  return kOk;
+}
+
+int ibcomm_hip_fabric_merge_counters(ibcomm_hip_fabric* fabric, uint64_t* launches_collected, uint64_t* launches_recorded) {
+  if (!fabric) return Fail(kInvalidArgument, "fabric is null");
+  if (launches_collected) *launches_collected = fabric->collector.collected();
+  if (launches_recorded) *launches_recorded = fabric->collector.issued();
+  return kOk;
+}
+
+int ibcomm_hip_fabric_set_merge_mode(ibcomm_hip_fabric* fabric, int mode) {
+  if (!fabric) return Fail(kInvalidArgument, "fabric is null");
+  if (mode != 0 && mode != 1) return Fail(kInvalidArgument, "merge mode must be 0 or 1");
+  if (mode != fabric->merge_mode) {
+    fabric->DropGraphs();  // recorded under the other setting
+    fabric->has_last_eager = false;
+  }
+  fabric->merge_mode = mode;
   return kOk;
 }
 

@@ -48,6 +48,7 @@
 
 #include "loopback.hpp"
 #include "memory_pool.hpp"
+#include "merge.hpp"
 #include "plan.hpp"
 #include "segments.hpp"
 #include "status.hpp"
@@ -152,6 +153,9 @@ class Communicator {
   int world_size() const { return world_size_; }
   MemoryPool<B>& pool() { return pool_; }
   Fabric<B>* fabric() { return fabric_; }
+  // While set, launches go to the collector instead of the stream (merge.hpp): for the recording of a
+  // whole world, where every rank issues on the one recording stream.
+  void set_collector(LaunchCollector<B>* c) { collector_ = c; }
   void set_max_fuse(int f) { max_fuse_ = f < 1 ? 1 : (f > kMaxSegments ? kMaxSegments : f); }
   void set_landing(int mode) { landing_ = mode; }
   int landing() const { return landing_; }
@@ -216,7 +220,7 @@ class Communicator {
       if (!in_place_ && bytes) {
         Stream s;
         IBCOMM_RETURN_IF_ERROR(pool_.NextStream(&s));
-        IBCOMM_RETURN_IF_ERROR(B::CopyAsync(recvbuf_, sendbuf_, bytes, s));
+        IBCOMM_RETURN_IF_ERROR(DeviceCopy(recvbuf_, sendbuf_, bytes, s));
         stats_.gather_copies++;
         stats_.gather_bytes += bytes;
       }
@@ -604,6 +608,7 @@ class Communicator {
   // them: the span is then the kernel's duration, without the few microseconds it costs the
   // device to process a marker before and after it.
   int LaunchTimed(const SegmentBatch& batch, Stream s, int role, Trace::DeviceCategory category) {
+    if (collector_) return collector_->Add(batch, dtype_, s);
     if (!DeviceTiming()) return B::LaunchSegments(batch, dtype_, s, role);
     DeviceSpan span;
     span.category = category;
@@ -796,7 +801,7 @@ class Communicator {
     for (int i = 0; i < batch.count; i++) {
       const Segment& seg = batch.seg[i];
       IBCOMM_RETURN_IF_ERROR(SpanBegin(s, Trace::kDeviceCopy));
-      IBCOMM_RETURN_IF_ERROR(B::CopyAsync(seg.dst, seg.a, seg.n * es_, s));
+      IBCOMM_RETURN_IF_ERROR(DeviceCopy(seg.dst, seg.a, seg.n * es_, s));
       IBCOMM_RETURN_IF_ERROR(SpanEnd(s));
       (*issued)++;
     }
@@ -927,7 +932,14 @@ class Communicator {
   // While this rank's traffic is being recorded for replay, keep a copy of the message's payload.
   int RecordPayload(const Message& m, Stream s) {
     if (!m.record_to) return kOk;
-    return B::CopyAsync(m.record_to, m.src, m.bytes, s);
+    return DeviceCopy(m.record_to, m.src, m.bytes, s);
+  }
+
+  // A device copy goes straight to the stream: whatever a collector still holds was issued before it
+  // and has to be on the stream first.
+  int DeviceCopy(void* dst, const void* src, size_t bytes, Stream s) {
+    if (collector_) IBCOMM_RETURN_IF_ERROR(collector_->Flush());
+    return B::CopyAsync(dst, src, bytes, s);
   }
 
   int CheckPeer(int peer) {
@@ -967,6 +979,7 @@ class Communicator {
   int rank_ = -1;
   MemoryPool<B> pool_;
   MemoryController<B> controller_;
+  LaunchCollector<B>* collector_ = nullptr;
   int max_fuse_ = kMaxSegments;
   int landing_ = kLandStaged;
   long long work_gpu_memory_size_ = 0;

@@ -155,16 +155,23 @@ class Fabric {
   // ranks in.  BeginSweep() freezes, for every channel, the set of receivable messages to those
   // posted so far; messages posted during the sweep become receivable at the next BeginSweep().
   // EndLockstep() lifts the limit (the threaded, one-thread-per-rank use never sets it).
+  // Completions are frozen the same way: a rank learns that a peer has taken its message at the
+  // next sweep, not from a peer the driver happened to visit earlier in this one.  (Otherwise the
+  // rank visited last would get its staging slots back a step before everybody else and write, in
+  // this step, into slots the first rank's launch of this step reads; correct on an in-order
+  // stream, but it keeps the two launches from being merged.)
   void BeginSweep() {
     for (auto& c : channels_) {
       std::lock_guard<std::mutex> lock(c->mu);
       c->visible_below = c->next_ticket;
+      c->completions_visible = c->completions.size();
     }
   }
   void EndLockstep() {
     for (auto& c : channels_) {
       std::lock_guard<std::mutex> lock(c->mu);
       c->visible_below = UINT64_MAX;
+      c->completions_visible = SIZE_MAX;
     }
   }
 
@@ -193,9 +200,10 @@ class Fabric {
   bool PollSendCompletion(int from, int to, Completion* out) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
-    if (c.completions.empty()) return false;
+    if (c.completions.empty() || c.completions_visible == 0) return false;
     *out = c.completions.front();
     c.completions.pop_front();
+    if (c.completions_visible != SIZE_MAX) c.completions_visible--;
     return true;
   }
 
@@ -203,9 +211,10 @@ class Fabric {
   size_t PollSendCompletions(int from, int to, std::vector<Completion>* out) {
     Channel& c = chan(from, to);
     std::lock_guard<std::mutex> lock(c.mu);
-    const size_t n = c.completions.size();
-    out->insert(out->end(), c.completions.begin(), c.completions.end());
-    c.completions.clear();
+    const size_t n = c.completions.size() < c.completions_visible ? c.completions.size() : c.completions_visible;
+    out->insert(out->end(), c.completions.begin(), c.completions.begin() + n);
+    c.completions.erase(c.completions.begin(), c.completions.begin() + n);
+    if (c.completions_visible != SIZE_MAX) c.completions_visible -= n;
     return n;
   }
 
@@ -315,6 +324,7 @@ class Fabric {
       std::lock_guard<std::mutex> lock(c->mu);
       c->inbox.clear();
       c->completions.clear();
+      if (c->completions_visible != SIZE_MAX) c->completions_visible = 0;
     }
     std::lock_guard<std::mutex> lock(poison_mu_);
     poisoned_.store(false);
@@ -347,6 +357,7 @@ class Fabric {
     std::deque<Completion> completions;
     uint64_t next_ticket = 0;
     uint64_t visible_below = UINT64_MAX;
+    size_t completions_visible = SIZE_MAX;  // how many of `completions`, from the front, the sender may see (lockstep sweeps)
     uint64_t posted = 0;
     uint64_t taken = 0;
     uint64_t delivered = 0;

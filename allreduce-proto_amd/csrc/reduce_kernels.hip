@@ -284,7 +284,7 @@ hipError_t Prepare(const SegmentBatch& given, int dtype, SegmentBatch* batch, La
   shape->die_local = tiles >= 64 && tiles <= kDieLocalMaxTiles;
   // Stores go through the memory-side cache while a launch writes at most half of its 256 MB
   // (config 2's ring step writes 32 MiB, config 5's 64 MiB; config 3's first halving step 192 MiB).
-  shape->write_through = written <= (uint64_t(128) << 20);
+  shape->write_through = written <= kWriteThroughMaxBytes;
   return hipSuccess;
 }
 

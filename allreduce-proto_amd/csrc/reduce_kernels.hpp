@@ -45,6 +45,10 @@
 
 namespace ibcomm_hip {
 
+// A launch's stores carry sc1 while it writes at most this many bytes, the non-temporal hint beyond (half of
+// the 256 MB cache in front of HBM; see the kernels' source for the measurements).
+constexpr uint64_t kWriteThroughMaxBytes = uint64_t(128) << 20;
+
 // How a launch will be issued, for tests and the benchmark's report.
 struct LaunchShape {
   bool aligned;    // AlignedSegmentKernel (true) or SegmentKernel (false)

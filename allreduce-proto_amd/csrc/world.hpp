@@ -21,9 +21,12 @@ namespace ibcomm_hip {
 // Issues one allreduce on every rank.  With `synchronize` the call returns when all results are in
 // place (the reference's blocking semantics); without it only the host-side issue is done and the
 // caller synchronises (used while recording a graph).
+// With a `collector` (only where all ranks issue on one stream, i.e. while a world is being recorded) the
+// ranks' launches are merged as far as their memory accesses allow (merge.hpp); everything
+// collected is on the stream when the call returns.
 template <class B>
 int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const void* const* sendbufs,
-             void* const* recvbufs, size_t len_elements, bool synchronize) {
+             void* const* recvbufs, size_t len_elements, bool synchronize, LaunchCollector<B>* collector = nullptr) {
   if (n < 1) return Fail(kInvalidArgument, "empty world");
   for (int r = 0; r < n; r++) {
     if (comms[r]->world_size() != n || comms[r]->rank() != r)
@@ -32,6 +35,7 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
   }
   int rc = kOk;
   int begun = 0;
+  for (int r = 0; r < n; r++) comms[r]->set_collector(collector);
   for (; begun < n; begun++) {
     rc = comms[begun]->Begin(algo, dtype, sendbufs[begun], recvbufs[begun], len_elements);
     if (rc != kOk) break;
@@ -65,6 +69,11 @@ int RunWorld(Communicator<B>* const* comms, int n, int algo, int dtype, const vo
     }
   }
   comms[0]->fabric()->EndLockstep();
+  for (int r = 0; r < n; r++) comms[r]->set_collector(nullptr);
+  if (collector) {
+    if (rc == kOk) rc = collector->Flush();
+    else collector->Discard();
+  }
   if (rc != kOk) {
     // keep the message of the first failure
     char saved[512];

@@ -31,6 +31,7 @@ EXPORTS = [
     "ibcomm_hip_send", "ibcomm_hip_recv", "ibcomm_hip_send_poll", "ibcomm_hip_recv_poll", "ibcomm_hip_send_wait",
     "ibcomm_hip_recv_wait", "ibcomm_hip_bcast", "ibcomm_hip_comm_set_trace", "ibcomm_hip_comm_set_timer_base", "ibcomm_hip_comm_dump_trace",
     "ibcomm_hip_world_allreduce_noalloc", "ibcomm_hip_describe_launch", "ibcomm_hip_copy_segments",
+    "ibcomm_hip_fabric_set_merge_mode", "ibcomm_hip_fabric_merge_counters",
 ]
 
 
@@ -87,6 +88,8 @@ def lib():
     L.ibcomm_hip_plan_send.argtypes = [vp, i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
     L.ibcomm_hip_fabric_set_graph_mode.argtypes = [vp, i]
     L.ibcomm_hip_fabric_graph_counters.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+    L.ibcomm_hip_fabric_set_merge_mode.argtypes = [vp, i]
+    L.ibcomm_hip_fabric_merge_counters.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
     L.ibcomm_hip_comm_set_max_fuse.argtypes = [vp, i]
     L.ibcomm_hip_comm_set_landing.argtypes = [vp, i]
     L.ibcomm_hip_comm_stats.argtypes = [vp, C.POINTER(Stats)]
@@ -192,6 +195,15 @@ class World:
         a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
         assert lib().ibcomm_hip_fabric_graph_counters(self.fabric, C.byref(a), C.byref(b), C.byref(c)) == 0
         return a.value, b.value, c.value
+
+    def set_merge_mode(self, mode):
+        assert lib().ibcomm_hip_fabric_set_merge_mode(self.fabric, mode) == 0, last_error()
+
+    def merge_counters(self):
+        """-> (launches the ranks handed in while worlds were recorded, launches recorded after merging)."""
+        a, b = C.c_uint64(), C.c_uint64()
+        assert lib().ibcomm_hip_fabric_merge_counters(self.fabric, C.byref(a), C.byref(b)) == 0
+        return a.value, b.value
 
     def set_max_fuse(self, f):
         for h in self.comms:

@@ -162,6 +162,16 @@ int ibcomm_hip_fabric_set_graph_mode(ibcomm_hip_fabric* fabric, int mode);
 int ibcomm_hip_fabric_graph_counters(ibcomm_hip_fabric* fabric, uint64_t* eager_calls, uint64_t* captures,
                                      uint64_t* replays);
 
+/* While a whole world is recorded, the launches the ranks issue for one step of the algorithm --
+ * independent of one another, what N devices would run side by side -- are merged into one launch
+ * as far as their memory accesses allow, so that a replay pays one kernel boundary per step instead
+ * of one per rank and step (8 ranks, ring: 14 launches instead of 112).  Results are unchanged bit
+ * for bit.  mode 0 turns that off, mode 1 is the default (IBCOMM_HIP_MERGE_RANKS); the counters say
+ * how many launches the ranks handed in during recordings and how many were recorded.  No
+ * counterpart in the reference, where every rank is a process with a device of its own. */
+int ibcomm_hip_fabric_set_merge_mode(ibcomm_hip_fabric* fabric, int mode);
+int ibcomm_hip_fabric_merge_counters(ibcomm_hip_fabric* fabric, uint64_t* launches_collected, uint64_t* launches_recorded);
+
 /* The reduction kernel on its own, asynchronous on `stream` (a hipStream_t, NULL = default
  * stream): dst[i] = a[i] + b[i].  Stands for _reduce_inplace_cuda<T>
  * (ibcomm/allreduce_cuda_impl.h:26-33, launches at :132-133 and :510-512), which is the case

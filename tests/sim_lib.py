@@ -24,7 +24,8 @@ class EngineStats(C.Structure):
 
 class Report(C.Structure):
     _fields_ = [("rc", C.c_int), ("nodes", C.c_long), ("races", C.c_long), ("unrecorded_waits", C.c_long),
-                ("rank0", EngineStats), ("error", C.c_char * 512), ("first_race", C.c_char * 256)]
+                ("rank0", EngineStats), ("error", C.c_char * 512), ("first_race", C.c_char * 256),
+                ("launches_collected", C.c_long), ("launches_issued", C.c_long)]
 
 
 _lib = None
@@ -50,7 +51,8 @@ def allreduce(algo, sendbufs, chunksize=None, max_fuse=48, landing=0, seed=0, th
               pool_bytes=1 << 16, in_place=False, streams=None, copy=True):
     """-> (rc, [recvbuf per rank], Report).  Environment knobs are set for the duration of the call.
     threaded: False = one thread steps all ranks, True (1) = one thread per rank, each with its own engine,
-    2 = one thread per rank, the blocking calls meet and the last to arrive steps all ranks."""
+    2 = one thread per rank, the blocking calls meet and the last to arrive steps all ranks, 3 = one thread, all ranks
+    on one stream with their launches merged across ranks (a recording of a world)."""
     world = len(sendbufs)
     if copy:  # copy=False: run on the caller's arrays, whatever their alignment
         sendbufs = [np.ascontiguousarray(s).copy() for s in sendbufs]

@@ -52,7 +52,8 @@ int main(int argc, char** argv) {
       rp[i] = recv[i].data();
     }
     const int fuse = (rng() % 2) ? 64 : 1 + rng() % 64, landing = rng() % 4;
-    const int threaded = (all_threaded || rng() % 5 == 0) ? 1 + it % 2 : 0;
+    // single-threaded worlds: every third one issues on one stream with its ranks' launches merged, as a recording does
+    const int threaded = (all_threaded || rng() % 5 == 0) ? 1 + it % 2 : (it % 3 == 0 ? 3 : 0);
     int rc = sim_world_allreduce(algo, 0, world, sp.data(), rp.data(), n, fuse, landing, it, threaded, 1 + rng() % 2, report);
     runs++;
     if (rc != 0) {

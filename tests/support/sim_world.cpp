@@ -27,11 +27,14 @@ struct sim_report {
   EngineStats rank0;
   char error[512];
   char first_race[256];
+  long launches_collected;  // threaded == 3: launches the ranks handed to the collector ...
+  long launches_issued;     // ... and launches it put on the stream
 };
 
 // threaded = 0: one thread steps all ranks (RunWorld); 1: one thread per rank, each running its own
 // engine (AllreduceBlocking); 2: one thread per rank, the calls meet and the last to arrive steps all
-// ranks (Rendezvous, what the library's blocking per-rank entry points do).
+// ranks (Rendezvous, what the library's blocking per-rank entry points do); 3: one thread steps all ranks, all
+// of them issuing on ONE stream with their launches merged across ranks (what a recording of a world does).
 // repeats > 1 runs the same collective again on the same communicators (event/slot reuse).
 int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendbufs, void* const* recvbufs, size_t len,
                         int max_fuse, int landing, unsigned seed, int threaded, int repeats, sim_report* rep) {
@@ -50,8 +53,17 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
     raw.push_back(comms.back().get());
   }
   Rendezvous meet(world);
+  LaunchCollector<SimBackend> collector;
+  SimBackend::Stream one = nullptr;
   for (int k = 0; k < repeats && rc == kOk; k++) {
-    if (!threaded) {
+    if (threaded == 3) {
+      if (!one) SimBackend::StreamCreate(&one);
+      for (auto* c : raw) c->pool().OverrideStream(one);
+      rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, false, &collector);
+      for (auto* c : raw) c->pool().ClearOverride();
+      SimBackend::StreamSynchronize(one);
+      if (rc != kOk) snprintf(rep->error, sizeof rep->error, "%s", LastErrorBuffer());
+    } else if (!threaded) {
       rc = RunWorld<SimBackend>(raw.data(), world, algo, dtype, sendbufs, recvbufs, len, true);
       if (rc != kOk) snprintf(rep->error, sizeof rep->error, "%s", LastErrorBuffer());
     } else {
@@ -102,6 +114,9 @@ int sim_world_allreduce(int algo, int dtype, int world, const void* const* sendb
   rep->unrecorded_waits = Sim::Get().unrecorded_waits();
   if (!raw.empty()) rep->rank0 = raw[0]->stats();
   snprintf(rep->first_race, sizeof rep->first_race, "%s", first.c_str());
+  rep->launches_collected = static_cast<long>(collector.collected());
+  rep->launches_issued = static_cast<long>(collector.issued());
+  if (one) SimBackend::StreamDestroy(one);
   return rc;
 }
 

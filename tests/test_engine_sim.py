@@ -111,6 +111,43 @@ def test_blocking_calls_of_all_ranks_meet_and_one_thread_drives(algo, world):
         assert rep.rank0.calls == 6
 
 
+@pytest.mark.parametrize("landing", [0, 1, 2, 3])
+@pytest.mark.parametrize("algo,world", [(RING, 2), (RING, 5), (RING, 8), (RABEN, 4), (RABEN, 16)])
+def test_launches_of_the_ranks_merge_while_a_world_is_recorded(algo, world, landing):
+    # every rank issues on one stream, as while a world is recorded, and hands its launches to the collector:
+    # launches that touch no common memory become one.  Bit-exact, free of conflicting accesses inside a
+    # launch (the simulator checks the segments of one launch against one another), twice in a row.
+    bufs = rand_bufs(world, 64 * 4 * world, seed=31)
+    rep = check(algo, bufs, 256, max_fuse=64, landing=landing, threaded=3, repeats=2, pool_bytes=1 << 20, seed=landing)
+    steps = 2 * (world - 1) if algo == RING else 2 * int(np.log2(world))
+    per_call = rep.launches_issued // 2
+    if landing in (2, 3):
+        # nothing but the algorithm's own steps is left: one launch per step, whatever the number of ranks
+        assert per_call == steps, (per_call, steps, rep.launches_collected)
+    if landing == 0:
+        assert rep.launches_issued <= rep.launches_collected  # reductions merge, the device copies stay
+    if landing == 1:
+        # a rank's landing copy and the reduction that reads it stay in order: the adds of a step merge, the copies do not
+        assert steps < per_call < rep.launches_collected // 2
+
+
+def test_merged_launches_on_random_shapes():
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        algo = int(rng.integers(0, 2))
+        world = int(rng.choice([2, 4, 8, 16])) if algo == RABEN else int(rng.integers(2, 10))
+        n = int(rng.integers(world, 5000))
+        chunk = None
+        if rng.random() < 0.6:
+            epc = int(rng.integers(1, max(2, n // (2 * world) + 1)))
+            if -(-n // epc) >= 2 * world:
+                chunk = 4 * epc
+        bufs = [(np.random.default_rng(case * 50 + r).standard_normal(n) * 9).astype(np.float32) for r in range(world)]
+        in_place = bool(rng.random() < 0.2)  # (a second call in place would add up the first one's results)
+        check(algo, bufs, chunk, max_fuse=int(rng.integers(1, 65)), landing=int(rng.integers(0, 4)), seed=case, threaded=3,
+              repeats=1 if in_place else int(rng.integers(1, 3)), pool_bytes=int(rng.choice([512, 4096, 65536])), in_place=in_place)
+
+
 def test_meeting_of_blocking_calls_handles_failures():
     held = S.lib().sim_rendezvous()
     names = ["five rounds, one driver each", "disagreeing ranks are all told", "a failed collective reaches every rank",

@@ -212,6 +212,49 @@ def test_graph_replays_match_eager_results(algo, world_size, chunk, landing):
         assert w.graph_counters()[0] == eager + 3
 
 
+@pytest.mark.parametrize("landing", [H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
+@pytest.mark.parametrize("algo,world_size,n,chunk", [(H.RING, 8, 1 << 20, 1 << 17), (H.RING, 5, 300007, None), (H.RABENSEIFNER, 16, 1 << 20, 1 << 14),
+                                                     (H.RABENSEIFNER, 4, 70001, None)])
+def test_recorded_world_merges_the_ranks_launches(algo, world_size, n, chunk, landing):
+    # While a world is recorded the launches the ranks issue for one step are merged into one as far as their
+    # memory accesses allow.  Replays of the merged graph, of the unmerged one and the eager call must agree
+    # bit for bit with the oracle, on fresh inputs each time; the counters show that merging happened.
+    host = [rand_bufs(world_size, n, seed=100 + k, scale=0.1) for k in range(4)]
+    results = {}
+    for merge in (1, 0):
+        with H.World(world_size) as w:
+            w.set_landing(landing)
+            w.set_merge_mode(merge)
+            send = G.to_device(host[0])
+            recv = [G.poisoned_like(t) for t in send]
+            got = []
+            for k in range(4):
+                for t, h in zip(send, host[k]):
+                    t.copy_(torch.from_numpy(h))
+                for t in recv:
+                    t.view(torch.uint8).fill_(0x55)
+                assert G.run_world(w, algo, send, recv, chunk) == 0, H.last_error()
+                got.append([t.clone() for t in recv])
+            assert w.graph_counters() == (1, 1, 3)
+            collected, recorded = w.merge_counters()
+            results[merge] = got
+            steps = 2 * (world_size - 1) if algo == H.RING else 2 * (world_size.bit_length() - 1)
+            if merge:
+                assert collected >= world_size * steps
+                if landing != H.LAND_KERNEL:
+                    assert recorded == steps, (collected, recorded)  # one launch per step of the algorithm
+                else:
+                    assert recorded < collected
+            else:
+                assert (collected, recorded) == (0, 0)
+    for k in range(4):
+        orc, want, _ = O.allreduce(G.ORACLE_ALGO[algo], host[k], chunk)
+        assert orc == 0
+        for r in range(world_size):
+            assert np.array_equal(O.bits(results[1][k][r].cpu().numpy()), O.bits(want[r])), (k, r)
+            assert G.bits_equal(results[1][k][r], results[0][k][r]), (k, r)
+
+
 @pytest.mark.parametrize("landing", [H.LAND_MEMCPY, H.LAND_KERNEL, H.LAND_DIRECT, H.LAND_STAGED])
 @pytest.mark.parametrize("algo,world_size,chunk", [(H.RING, 8, 65536), (H.RING, 3, None), (H.RABENSEIFNER, 8, 65536)])
 def test_one_rank_replayed_against_recorded_peers(algo, world_size, chunk, landing):
