@@ -6,8 +6,9 @@
 // "device memory" is a fixed array that lives in the library's code object, whose only stream is the
 // caller's, and whose events are nothing at all: every launch of every emulated rank is enqueued on
 // the one stream in the dependency-respecting order the single-threaded driver issues them in, and
-// an in-order stream then carries every ordering an event would have carried.  The call makes no
-// hipMalloc, hipFree, stream or event creation, and does not wait for the device.
+// an in-order stream then carries every ordering an event would have carried (and launches of
+// different ranks that touch no common memory are merged into one, as in a recorded world).  The
+// call makes no hipMalloc, hipFree, stream or event creation, and does not wait for the device.
 //
 // Every call on a GPU uses that GPU's copy of the array and finds the previous call's staging data
 // in it.  Nothing has to start at zero: a staging slot is written in full by the launch that
@@ -164,7 +165,10 @@ extern "C" int ibcomm_hip_world_allreduce_noalloc(int world_size, int algo, int 
       comms.back()->trace().Enable(false);
       cs.push_back(comms.back().get());
     }
-    if (rc == kOk) rc = RunWorld<StaticBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len_elements, false);
+    // one in-order stream for all ranks: their launches of one step merge as in a recorded world (merge.hpp)
+    LaunchCollector<StaticBackend> collector;
+    collector.set_write_limit(kWriteThroughMaxBytes);
+    if (rc == kOk) rc = RunWorld<StaticBackend>(cs.data(), world_size, algo, dtype, sendbufs, recvbufs, len_elements, false, &collector);
   }
   t_arena = nullptr;
   return rc;
