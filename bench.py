@@ -387,7 +387,7 @@ def print_variant_table(title, times, bytes_per_launch):
 
 
 def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
-    """Where one blocking call of the rank's schedule spends its time, from the library's trace: per-launch device
+    """Where one blocking call of the rank's schedule spends its time, from the library's trace: the launches' own
     durations when the call is issued eagerly, and for graph replays the host spans "graph launched" and "waiting for
     the completion flag" next to the device's first-kernel-to-end duration."""
     import statistics as st
@@ -434,7 +434,7 @@ def call_breakdown(torch, H, w, rank, algo, send_ptr, out_ptr, n):
     t, lines = traced(30)
     red, cp = lines["device-redu-kernel"][1::2], lines["device-copy-kernel"][1::2]
     per_call_red, per_call_cp = len(red) // 30, len(cp) // 30
-    print("eager issue, trace on:   %8.2f us per call; device durations between the HIP events around each launch:" % t)
+    print("eager issue, trace on:   %8.2f us per call; the launches' own durations (each leaves its begin and end timestamps in the trace):" % t)
     print("    %d reduction launches per call: median %.2f us, sum per call %.2f us" % (per_call_red, st.median(red) * 1e3, sum(red) / 30 * 1e3))
     print("    %d copy launches per call:      median %.2f us, sum per call %.2f us" % (per_call_cp, st.median(cp) * 1e3, sum(cp) / 30 * 1e3))
     issue = [lines[k][1::2] for k in ("issue-redu-kernel", "issue-copy-kernel", "issue-send", "received", "issue-recv", "reduced", "other")]
