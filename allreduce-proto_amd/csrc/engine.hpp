@@ -236,8 +236,11 @@ class Communicator {
     chunk_unconsumed_.assign(chunks, 0);
     chunk_pulled_.assign(chunks, OpState());
     chunk_in_batch_.assign(chunks, 0);
-    posted_.assign(world_size_, std::deque<PostedSend>());
-    arrived_.assign(world_size_, std::deque<Message>());
+    // per-peer queues are kept from call to call (a deque that is cleared keeps its first block)
+    posted_.resize(world_size_);
+    arrived_.resize(world_size_);
+    for (auto& q : posted_) q.clear();
+    for (auto& q : arrived_) q.clear();
     pending_reduce_.clear();
     pending_gather_.clear();
     // A slot needs spare bytes only if some chunk of recvbuf starts off a 16-byte boundary.  Without
