@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X allreduce hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5] [--no-others] [--all-configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5] [--no-others] [--all-configs] [--full]
     python bench.py --only-roofline [--config N]     the kernel leg alone (what the counter profiles run)
     python bench.py --whole-buffer                    adds roofline.whole_buffer_launch to the line
     python bench.py --sweep [--config N]              every kernel variant of the measurement library at the launch shape
@@ -732,6 +732,89 @@ def summary_of(res):
     return out
 
 
+def compact_leg(leg, top=True):
+    """A roofline leg without its prose: the contract's keys first, then the figures the measured table is made of.
+    `frac_into_recvbufs`: the same launches with the result walking through all recvbufs instead of the staging region;
+    `in_schedule_mean_us` / `_frac`: mean of the reduction launches' own begin-to-end times, issued one at a time in the
+    schedule's order (a replayed chain adds a kernel boundary per launch); `replay_device_us`: one replay of the rank's
+    schedule on the device, HIP events around the graph."""
+    out = {k: leg[k] for k in (("bound", "achieved", "peak", "unit", "frac", "traffic") if top else ("frac", "traffic")) if k in leg}
+    out["launch_shape"] = leg["launch_shape"]
+    if top:
+        out["algorithmic_bytes_per_launch"] = leg["algorithmic_bytes_per_launch"]
+    out["avg_launch_us"] = leg["avg_launch_us"]
+    out["target_0p80_met"] = leg.get("target_0p80_met")
+    out["frac_into_recvbufs"] = leg["result_walking_through_all_recvbufs"]["frac"]
+    for k, short in (("in_schedule_mean_us", "in_schedule_mean_us"), ("in_schedule_frac", "in_schedule_frac"), ("replay_device_us_per_call", "replay_device_us")):
+        if k in leg:
+            out[short] = leg[k]
+    if top and "in_schedule_mean_us" in leg:
+        out["in_schedule_is"] = "each launch's own time, issued alone in schedule order; a chain adds a kernel boundary"
+    return out
+
+
+def compact_line(full):
+    """The line that is printed by default: every figure, little prose.  (The driver that runs this benchmark keeps
+    only the end of its output, a few thousand characters; --full prints everything, with descriptions.)"""
+    full = dict(full)
+    full["metric"] = "emulated allreduce algbw, fp32 (+ reduce-kernel HBM roofline)"
+    line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                                 "vs_baseline", "dtype", "data")}
+    c = full["config"]
+    line["config"] = {"workload": "BASELINE configs[%d]: %s, %d emulated ranks x %d fp32, IBCOMM_CHUNKSIZE=%d; step = rank %d's complete schedule "
+                                  "on the GPU, peers replayed from a recording of the full world" % (
+                                      full["_config_id"] - 1, c["algo"], c["ranks"], c["elements_per_rank"], c["chunk_bytes"], c["measured_rank"]),
+                      "landing": c["landing"], "max_fuse": c["max_fuse"]}
+    line["parity_bit_exact"] = full["parity_bit_exact"]  # every configuration and landing mode of the run
+    e = full["extra"]
+
+    def landing(d):
+        return None if d is None else {k: d[k] for k in d if k != "parity_bit_exact"}
+
+    x = {"busbw_GBps": e["busbw_GBps"], "rank_device_GBps": e["rank_device_GBps"], "rank_frac_of_hbm_peak": e["rank_frac_of_hbm_peak"],
+         "rank_launches_per_step": e["rank_reduce_launches_per_step"] + e["rank_gather_launches_per_step"] + e["rank_landing_launches_per_step"],
+         "world_all_ranks_on_one_gpu": {k: e["world_all_ranks_on_one_gpu"][k] for k in ("ms_per_step", "algbw_GBps", "frac_of_hbm_peak")},
+         "rank_with_copy_kernel_landing": landing(e["rank_with_copy_kernel_landing"]),
+         "rank_with_hipMemcpyAsync_landing": landing(e["rank_with_hipMemcpyAsync_landing"]),
+         "issue": e["issue"], "graph_calls_eager_captured_replayed": e["graph_calls_eager_captured_replayed"],
+         "pool_slots_high_water": e["pool_slots_high_water"]}
+    if "other_configs" in e:
+        x["other_configs"] = {}
+        for name, o in e["other_configs"].items():
+            y = {"workload": o["workload"].replace(" allreduce, ", " ").replace(" emulated ranks, ", " x ").replace(" per rank, IBCOMM_CHUNKSIZE=", ", chunk "),
+                 "rank_ms_per_step": o["rank_ms_per_step"], "rank_algbw_GBps": o["rank_algbw_GBps"],
+                 "rank_frac_of_hbm_peak": o["rank_frac_of_hbm_peak"], "world_ms_per_step": o["world_all_ranks_on_one_gpu_ms_per_step"],
+                 "world_algbw_GBps": o["world_all_ranks_on_one_gpu_algbw_GBps"],
+                 "kernel_landing_rank_algbw_GBps": (o["rank_with_copy_kernel_landing"] or {}).get("algbw_GBps")}
+            if "roofline" in o:
+                y["roofline"] = compact_leg(o["roofline"], top=False)
+            x["other_configs"][name] = y
+    if "reference_api" in e:
+        x["reference_api"] = {"what": "8 rank threads in blocking IBVerbsCommunicator::AllreduceRingCuda<float> calls; 3 warm-ups, 10 timed; ms per allreduce"}
+        for name, o in e["reference_api"].items():
+            x["reference_api"][name] = o if "error" in o else {"first_timed_call": o["ms_per_allreduce_first_timed_call"], "median": o["ms_per_allreduce_median"],
+                                                               "max": o["ms_per_allreduce_max"], "all_ranks_ok": o["all_ranks_report_ok"]}
+    line["extra"] = x
+    if "roofline" in full:
+        r = full["roofline"]
+        leg = compact_leg(r)
+        leg["kernel"] = r["kernel"]
+        if "ceiling" in r:
+            leg["ceiling"] = {"best_of_57_other_forms_us": r["ceiling"]["best_variant_us"], "shipped_us_same_pass": r["ceiling"]["shipped_kernel_us_same_pass"],
+                              "shipped_over_best": r["ceiling"]["shipped_over_best"]}
+        if "whole_buffer_launch" in r:
+            leg["whole_buffer_launch"] = r["whole_buffer_launch"]
+        line["roofline"] = leg
+    if "cpu_baseline" in full:
+        b = full["cpu_baseline"]
+        line["cpu_baseline"] = {"value": b["value"], "unit": b["unit"], "cores": b["cores"], "kind": b["kind"],
+                                "sample": "same workload, whole; the oracle's restatement of AllreduceRing<float>, gcc -O2 scalar loop, one thread per rank, best of 15",
+                                "seconds": b["seconds"], "cpu_model": b["cpu_model"], "logical_cpus": b["logical_cpus"],
+                                "single_core_reduce_loop_GBps": b["single_core_reduce_loop_GBps"],
+                                "config1_ring_4x16MiB": {k: b["config1_ring_4x16MiB"][k] for k in ("seconds", "algbw_GBps", "equals_exact_integer_sum")}}
+    return line
+
+
 def reference_api_leg(cfg, timed_runs=10):
     """The reference's own entry point and timing protocol: one IBVerbsCommunicator per rank, one host thread per rank,
     every rank in a blocking AllreduceRingCuda / AllreduceRabenseifnerCuda call; 3 warm-ups, then timed runs
@@ -780,6 +863,7 @@ def main():
     ap.add_argument("--no-roofline", action="store_true", help="skip the kernel roofline leg")
     ap.add_argument("--no-others", action="store_true",
                     help="skip extra.other_configs (configurations 4 and 3 measured after the headline one) and extra.reference_api")
+    ap.add_argument("--full", action="store_true", help="print the line with every detail and description (several times longer)")
     ap.add_argument("--all-configs", action="store_true", help="extra.other_configs also holds configuration 5 (32 ranks x 2 GiB)")
     ap.add_argument("--only-roofline", action="store_true",
                     help="run only the kernel roofline leg at the workload's launch shape (for profiling the kernel alone)")
@@ -938,7 +1022,10 @@ def main():
         line["cpu_baseline"] = cpu_baseline_leg(O, world, n, chunk, algo_name)
         # the like-for-like GPU figure for that baseline: all N ranks' schedules on the one GPU per step
         line["cpu_baseline"]["gpu_all_ranks_on_one_gpu_algbw_GBps"] = round(world_algbw, 2)
-    print(json.dumps(line))
+    line["_config_id"] = args.config
+    out = line if args.full else compact_line(line)
+    out.pop("_config_id", None)
+    print(json.dumps(out, separators=(",", ":")) if not args.full else json.dumps(out))
     if not parity:
         sys.exit(1)
 
