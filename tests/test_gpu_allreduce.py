@@ -456,6 +456,37 @@ def test_config_3_rabenseifner_16_ranks_resnet50():
         assert st["reduce_elements"] == 90 * 1048576  # rank 0 reduces 90 chunks
 
 
+@pytest.mark.parametrize("cfg", [2, 3, 4])
+def test_full_size_configs_through_the_blocking_per_rank_calls(cfg):
+    # The reference's usage at the benchmark's sizes: one thread per rank, each in its blocking call; the calls meet,
+    # the world is issued eagerly, recorded with the ranks' launches merged, and replayed.  Four calls on fresh
+    # inputs; every element of every rank after every call, with torch's fp32 adds in the reference's order.
+    algo, world_size, n, chunk, kind = {2: (H.RING, 8, 67108864, 8388608, "normal"), 3: (H.RABENSEIFNER, 16, 102760448, 4194304, "normal1e-2"),
+                                        4: (H.RING, 8, 16777216, 65536, "uniform")}[cfg]
+    with G.env(IBCOMM_NUM_CUDA_STREAM=64 if cfg == 4 else None):
+        with H.World(world_size) as w:
+            send = device_inputs(world_size, n, 500 + cfg, kind)
+            recv = [G.poisoned_like(t) for t in send]
+            for call in range(4):
+                if call:
+                    for r, t in enumerate(send):  # fresh contents in the same buffers
+                        t.mul_(-0.5).add_(send[(r + 1) % world_size], alpha=0.25)
+                    for t in recv:
+                        t.view(torch.uint8).fill_(0x55)
+                assert G.run_world(w, algo, send, recv, chunk, threads=True) == 0, H.last_error()
+                if algo == H.RING:
+                    check_ring_on_device(send, recv, chunk)
+                else:
+                    want = G.device_tree(send, (0, n))
+                    for r in range(world_size):
+                        assert G.bits_equal(recv[r], want), "call %d rank %d" % (call, r)
+            assert w.graph_counters() == (1, 1, 3)
+            collected, recorded = w.merge_counters()
+            assert 0 < recorded < collected
+    if cfg == 4:
+        assert recorded == 14  # one launch per step of the ring for all 8 ranks
+
+
 def test_config_4_ring_small_chunks_64_streams():
     world_size, n, chunk = 8, 16777216, 65536
     with G.env(IBCOMM_NUM_CUDA_STREAM=64):
